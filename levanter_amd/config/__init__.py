@@ -2,6 +2,7 @@ from .lm_config import ConfigError, LmConfig
 from .gpt2 import Gpt2Config
 from .zederax import ZederaxConfig
 from .nakurax import NakuraxConfig
+from .tativik import TativikConfig
 from .engine_config import InferenceEngineConfig
 
-__all__ = ["ConfigError", "LmConfig", "Gpt2Config", "ZederaxConfig", "NakuraxConfig", "InferenceEngineConfig"]
+__all__ = ["ConfigError", "LmConfig", "Gpt2Config", "ZederaxConfig", "NakuraxConfig", "TativikConfig", "InferenceEngineConfig"]

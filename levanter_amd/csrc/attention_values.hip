@@ -13,6 +13,8 @@
 //   score(t, key) = cap(scale * q . k) - slope[h] * (position(t) - position(key)),  cap(s) = softcap * tanh(s / softcap)
 //   a query at position p sees keys max(0, p - window + 1) .. p (window 0: all) and, with chunk > 0, only keys of its own
 //   chunk of positions, (p / chunk) * chunk .. p (chunks are counted from position 0). A key whose block has no page is masked.
+//   sinks (float32 [H] or null): the softmax's denominator of head h also holds exp(sinks[h]), once per query: a score without
+//   a key and without a value, neither scaled nor capped.
 // One wave per (query token, head); keys are visited 64 at a time.
 #include "common.h"
 
@@ -24,7 +26,7 @@ __global__ void __launch_bounds__(64)
 attention_values_kernel(const T* __restrict__ q, long q_stride, float* __restrict__ out, const T* __restrict__ k_pages,
                         const T* __restrict__ v_pages, const int* __restrict__ positions, const int* __restrict__ token_seq,
                         const int* __restrict__ block_tables, int bt_stride, int H, int KVH, int HD, int VD, int NV, int PS, float scale,
-                        int window, int chunk, float softcap, const float* __restrict__ slopes) {
+                        int window, int chunk, float softcap, const float* __restrict__ slopes, const float* __restrict__ sinks) {
   __shared__ float qs[AV_MAX_HD];
   __shared__ float ps[64];
   __shared__ int pg[64];
@@ -89,6 +91,7 @@ attention_values_kernel(const T* __restrict__ q, long q_stride, float* __restric
     }
     __syncthreads();
   }
+  if (sinks != nullptr) l = m == -INFINITY ? 1.0f : l + expf(sinks[h] - m);
   const float inv = l > 0.f ? 1.0f / l : 0.f;
   float* o = out + ((size_t)t * H + h) * NV * VD + (size_t)c_first * VD;
 #pragma unroll
@@ -101,7 +104,7 @@ attention_values_kernel(const T* __restrict__ q, long q_stride, float* __restric
 extern "C" int lev_attention_values(const void* q, long q_stride, float* out, const void* k_pages, const void* v_pages,
                                     const int* positions, const int* token_seq, const int* block_tables, int bt_stride, int T, int H,
                                     int KVH, int HD, int VD, int NV, int PS, float scale, int window, int chunk, float softcap,
-                                    const float* slopes, int dtype, hipStream_t stream) {
+                                    const float* slopes, const float* sinks, int dtype, hipStream_t stream) {
   LEV_REQUIRE(T >= 0 && H > 0 && KVH > 0 && H % KVH == 0, "attention: bad head counts heads=%d kv_heads=%d", H, KVH);
   LEV_REQUIRE(HD > 0 && HD % 8 == 0 && HD <= AV_MAX_HD, "attention: head_dim=%d must be a multiple of 8 and at most %d", HD, AV_MAX_HD);
   LEV_REQUIRE(VD > 0 && (NV == 1 || NV == KVH), "attention: value size %d, value heads per query head %d (1 or kv_heads=%d)", VD, NV, KVH);
@@ -116,10 +119,10 @@ extern "C" int lev_attention_values(const void* q, long q_stride, float* out, co
   if (dtype == LEV_F32)
     attention_values_kernel<float><<<grid, 64, 0, stream>>>((const float*)q, q_stride, out, (const float*)k_pages, (const float*)v_pages,
                                                            positions, token_seq, block_tables, bt_stride, H, KVH, HD, VD, NV, PS, scale,
-                                                           window, chunk, softcap, slopes);
+                                                           window, chunk, softcap, slopes, sinks);
   else
     attention_values_kernel<bf16_t><<<grid, 64, 0, stream>>>((const bf16_t*)q, q_stride, out, (const bf16_t*)k_pages,
                                                             (const bf16_t*)v_pages, positions, token_seq, block_tables, bt_stride, H, KVH,
-                                                            HD, VD, NV, PS, scale, window, chunk, softcap, slopes);
+                                                            HD, VD, NV, PS, scale, window, chunk, softcap, slopes, sinks);
   return lev_check_launch("attention_values");
 }

@@ -20,6 +20,8 @@
 //
 //   score(t, key) = cap(scale * q . k) - slope[h] * (position(t) - position(key)),  cap(s) = softcap * tanh(s / softcap)
 //   out [T][H][NV][VD] float32, as attention_values.hip writes it.
+//   sinks (float32 [H] or null): exp(sinks[h]) is added to the denominator of head h's softmax, once per query (a token whose
+//   keys are split over waves gets it in the merge).
 #include "common.h"
 #include "attention_config.h"
 
@@ -63,7 +65,7 @@ attention_values_mfma_kernel(const bf16_t* __restrict__ q, long q_stride, float*
                              const bf16_t* __restrict__ v_pages, const int* __restrict__ positions, const int* __restrict__ token_seq,
                              const int* __restrict__ block_tables, int bt_stride, const int* __restrict__ work, int H, int KVH, int NV,
                              int PS, float scale, int window, int chunk, float softcap, const float* __restrict__ slopes, int splits,
-                             float* __restrict__ part_o, float* __restrict__ part_ml) {
+                             float* __restrict__ part_o, float* __restrict__ part_ml, const float* __restrict__ sinks) {
   const int lane = threadIdx.x, col = lane & 15, g = lane >> 4;
   const int group = H / KVH;
   int tok = 0, head = 0, kvh = 0;
@@ -227,6 +229,7 @@ attention_values_mfma_kernel(const bf16_t* __restrict__ q, long q_stride, float*
     }
     return;
   }
+  if (sinks != nullptr) l = m == -INFINITY ? 1.0f : l + __builtin_amdgcn_exp2f(sinks[head] * LOG2E - m);  // m is in base 2
   const float inv = l > 0.f ? 1.0f / l : 0.f;
 #pragma unroll
   for (int c = 0; c < NVC; ++c) {
@@ -251,7 +254,8 @@ __global__ void __launch_bounds__(PF_THREADS)
 attention_values_mfma_runs_kernel(const bf16_t* __restrict__ q, long q_stride, float* __restrict__ out, const bf16_t* __restrict__ k_pages,
                                   const bf16_t* __restrict__ v_pages, const int* __restrict__ positions, const int* __restrict__ token_seq,
                                   const int* __restrict__ block_tables, int bt_stride, const int* __restrict__ tiles, int H, int KVH, int NV,
-                                  int PS, float scale, int window, int chunk, float softcap, const float* __restrict__ slopes) {
+                                  int PS, float scale, int window, int chunk, float softcap, const float* __restrict__ slopes,
+                                  const float* __restrict__ sinks) {
   extern __shared__ __attribute__((aligned(16))) unsigned char av_smem[];
   bf16_t* ks = reinterpret_cast<bf16_t*>(av_smem);  // [HD/8][64][8]
   bf16_t* vs = ks + HD * 64;                        // [n_c][VD][VS_STRIDE]
@@ -435,6 +439,7 @@ attention_values_mfma_runs_kernel(const bf16_t* __restrict__ q, long q_stride, f
   l += __shfl_xor(l, 16, 64);
   l += __shfl_xor(l, 32, 64);
   if (!valid) return;
+  if (sinks != nullptr) l = m == -INFINITY ? 1.0f : l + __builtin_amdgcn_exp2f(sinks[head] * LOG2E - m);  // m is in base 2
   const float inv = l > 0.f ? 1.0f / l : 0.f;
 #pragma unroll
   for (int c = 0; c < NVC; ++c) {
@@ -450,7 +455,7 @@ attention_values_mfma_runs_kernel(const bf16_t* __restrict__ q, long q_stride, f
 #define MERGE_MAX_SPLITS 32
 __global__ void __launch_bounds__(64)
 attention_values_merge_kernel(const float* __restrict__ part_o, const float* __restrict__ part_ml, const int* __restrict__ singles,
-                              float* __restrict__ out, int H, int n_out, int splits) {
+                              float* __restrict__ out, int H, int n_out, int splits, const float* __restrict__ sinks) {
   __shared__ float w_s[MERGE_MAX_SPLITS + 8];
   const int idx = blockIdx.x, head = blockIdx.y, lane = threadIdx.x;
   // lane s holds split s's maximum and sum; loads stand under no condition (clamped index, the value replaced afterwards)
@@ -459,7 +464,8 @@ attention_values_merge_kernel(const float* __restrict__ part_o, const float* __r
   const float ms = lane < splits ? mv : -INFINITY;
   const float M = wave_max(ms);
   const float w = __builtin_amdgcn_exp2f(ms - (M == -INFINITY ? 0.f : M));  // a split without keys, a lane without a split: 0
-  const float L = wave_sum(w * (lane < splits ? lv : 0.f));
+  float L = wave_sum(w * (lane < splits ? lv : 0.f));
+  if (sinks != nullptr) L = M == -INFINITY ? 1.0f : L + __builtin_amdgcn_exp2f(sinks[head] * 1.4426950408889634f - M);
   if (lane < MERGE_MAX_SPLITS + 8) w_s[lane] = w;
   __syncthreads();
   const float inv = L > 0.f ? 1.0f / L : 0.f;
@@ -485,7 +491,7 @@ extern "C" int lev_attention_values_mfma(const void* q, long q_stride, float* ou
                                          const int* positions, const int* token_seq, const int* block_tables, int bt_stride,
                                          const int* tiles, int n_tiles, const int* singles, int n_singles, int H, int KVH, int HD_,
                                          int VD_, int NV, int PS, float scale, int window, int chunk, float softcap, const float* slopes,
-                                         int splits, float* workspace, int max_keys, hipStream_t stream) {
+                                         const float* sinks, int splits, float* workspace, int max_keys, hipStream_t stream) {
   LEV_REQUIRE(HD_ == HD && VD_ == VD, "attention: this library was built for head sizes %d / %d, not %d / %d", HD, VD, HD_, VD_);
   LEV_REQUIRE(H > 0 && KVH > 0 && H % KVH == 0, "attention: bad head counts heads=%d kv_heads=%d", H, KVH);
   LEV_REQUIRE(NV == 1 || NV == KVH, "attention: %d value heads per query head (1 or kv_heads=%d)", NV, KVH);
@@ -509,11 +515,11 @@ extern "C" int lev_attention_values_mfma(const void* q, long q_stride, float* ou
     if (lds + RUN_PAGES * sizeof(int) <= 64 * 1024 && reach / PS + 2 <= RUN_PAGES)
       attention_values_mfma_runs_kernel<<<grid, PF_THREADS, lds, stream>>>((const bf16_t*)q, q_stride, out, (const bf16_t*)k_pages,
                                                                          (const bf16_t*)v_pages, positions, token_seq, block_tables,
-                                                                         bt_stride, tiles, H, KVH, NV, PS, scale, window, chunk, softcap, slopes);
+                                                                         bt_stride, tiles, H, KVH, NV, PS, scale, window, chunk, softcap, slopes, sinks);
     else  // the largest head sizes, the longest ranges: every wave by itself, operands straight from the pages
       attention_values_mfma_kernel<false><<<dim3(n_tiles * SUB_TILES, H, chunks), 64, 0, stream>>>(
           (const bf16_t*)q, q_stride, out, (const bf16_t*)k_pages, (const bf16_t*)v_pages, positions, token_seq, block_tables, bt_stride,
-          tiles, H, KVH, NV, PS, scale, window, chunk, softcap, slopes, 1, nullptr, nullptr);
+          tiles, H, KVH, NV, PS, scale, window, chunk, softcap, slopes, 1, nullptr, nullptr, sinks);
     if (lev_check_launch("attention_values_mfma (runs)")) return -1;
   }
   if (n_singles > 0) {
@@ -524,10 +530,10 @@ extern "C" int lev_attention_values_mfma(const void* q, long q_stride, float* ou
     attention_values_mfma_kernel<true><<<grid, 64, 0, stream>>>((const bf16_t*)q, q_stride, out, (const bf16_t*)k_pages,
                                                                (const bf16_t*)v_pages, positions, token_seq, block_tables, bt_stride,
                                                                singles, H, KVH, NV, PS, scale, window, chunk, softcap, slopes, splits, part_o,
-                                                               part_ml);
+                                                               part_ml, sinks);
     if (lev_check_launch("attention_values_mfma (single tokens)")) return -1;
     if (splits > 1) {
-      attention_values_merge_kernel<<<dim3(n_singles, H), 64, 0, stream>>>(part_o, part_ml, singles, out, H, NV * VD, splits);
+      attention_values_merge_kernel<<<dim3(n_singles, H), 64, 0, stream>>>(part_o, part_ml, singles, out, H, NV * VD, splits, sinks);
       if (lev_check_launch("attention_values_mfma (merge)")) return -1;
     }
   }

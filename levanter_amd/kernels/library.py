@@ -73,6 +73,18 @@ class PendingStreams:
         self.out, self.streams, self.y, self.mix, self.w_out, self.y_pending = out, streams, y, mix, w_out, y_pending
 
 
+class PendingGatedNorm:
+    """A sublayer's result ``y`` (float32 ``[T, D]``) that has not been added to the residual stream ``out`` yet
+    (``HipKernels.group_norm_step`` with ``defer``): ``out`` still lacks ``mult * gn(y * sigmoid(gate), post_weight)`` with
+    ``gn`` the RMS norm in ``groups`` groups. The next ``group_norm_step`` that reads ``out`` does it in its own pass;
+    ``HipKernels.finish`` runs it by itself."""
+
+    __slots__ = ("out", "y", "gate", "post_weight", "mult", "groups", "eps")
+
+    def __init__(self, out, y, gate, post_weight, mult, groups, eps):
+        self.out, self.y, self.gate, self.post_weight, self.mult, self.groups, self.eps = out, y, gate, post_weight, mult, groups, eps
+
+
 def _ptr(t: Optional[torch.Tensor]):
     """A tensor's address as ctypes takes it for a ``c_void_p`` parameter: a plain integer, or None."""
     return None if t is None else t.data_ptr()
@@ -239,6 +251,9 @@ class HipKernels:
             _req(n == x.shape[0], "norm: out must have as many rows as x")
         else:
             _req(rows.dtype == torch.int32 and rows.numel() == n, "norm: rows must be int32, one per output row")
+        if isinstance(pending, PendingGatedNorm):  # another kind of norm behind a gated sublayer: finish that first
+            self.finish(pending)
+            pending = None
         if isinstance(pending, PendingStreams):
             _req(pending.out is x, "norm: the unfinished streams belong to another tensor")
             if rms and bias is None and D * 4 <= 60 * 1024:
@@ -291,6 +306,9 @@ class HipKernels:
         """Finish a product that ``linear(..., may_leave_pending=True)`` left unfinished, or a deferred sum of streams."""
         if isinstance(pending, PendingStreams):
             self.streams_step(pending.streams, y=pending.y, mix=pending.mix, w_out=pending.w_out, x_out=pending.out, y_pending=pending.y_pending)
+            return
+        if isinstance(pending, PendingGatedNorm):
+            self.group_norm_step(pending.out, groups=pending.groups, eps=pending.eps, pending=pending)
             return
         if isinstance(pending, PendingProduct):
             x = pending.out
@@ -550,14 +568,15 @@ class HipKernels:
 
     def attention_values(self, q, out, k_pages, v_pages, meta, *, n_heads: int, n_kv_heads: int, head_dim: int, value_dim: int,
                          all_value_heads: bool, page_size: int, scale: float, window: Optional[int], block_tables,
-                         softcap: Optional[float] = None, slopes=None, chunk: Optional[int] = None) -> None:
+                         softcap: Optional[float] = None, slopes=None, chunk: Optional[int] = None, sinks=None) -> None:
         """Causal attention over the pages for heads whose keys and values differ in size. ``out`` float32
         [T, heads, NV, value_dim]: the weights of each query head applied to the values of every key/value head
         (``all_value_heads``: NV = kv heads, for weights that are mixed over the heads afterwards, see ``head_talk``) or of its
         own (NV = 1). Score: ``cap(scale q.k) - slopes[h] * distance`` (``slopes`` float32 [heads] or None), ``cap`` the soft
         cap if given. ``chunk``: a query sees only the keys of its own chunk of that many positions, counted from position 0.
+        ``sinks`` (float32 [heads] or None): the denominator of head h's softmax also holds ``exp(sinks[h])``, once per query.
         The cache must hold the step's own keys and values already."""
-        _dev(q, out, k_pages, v_pages, block_tables, meta.positions, meta.token_seq, slopes)
+        _dev(q, out, k_pages, v_pages, block_tables, meta.positions, meta.token_seq, slopes, sinks)
         T = q.shape[0]
         dt = q.dtype
         nv = n_kv_heads if all_value_heads else 1
@@ -568,6 +587,7 @@ class HipKernels:
         _req(k_pages.is_contiguous() and v_pages.is_contiguous() and k_pages.numel() * value_dim == v_pages.numel() * head_dim
              and k_pages.numel() % (n_kv_heads * head_dim * page_size) == 0, "attention_values: page tensors do not fit the sizes")
         _req(slopes is None or (slopes.dtype == torch.float32 and slopes.numel() == n_heads and slopes.is_contiguous()), "attention_values: one float32 slope per head")
+        _req(sinks is None or (sinks.dtype == torch.float32 and sinks.numel() == n_heads and sinks.is_contiguous()), "attention_values: one float32 sink per head")
         if dt == torch.bfloat16 and self.use_mfma and self.mfma_attention_values_supports(head_dim, value_dim):
             # matrix cores: runs of several tokens in tiles of 16 query rows, single tokens with the heads of a key/value head as columns
             lib = self._unit(_build.attention_values_unit(head_dim, value_dim))
@@ -593,12 +613,12 @@ class HipKernels:
                 _ptr(q), _rows(q, "attention_values: q"), _ptr(out), _ptr(k_pages), _ptr(v_pages), _ptr(meta.positions), _ptr(meta.token_seq),
                 _ptr(block_tables), block_tables.shape[1], _ptr(meta.prefill_tiles), meta.n_prefill_tiles, _ptr(meta.decode_tokens),
                 meta.n_decode, n_heads, n_kv_heads, head_dim, value_dim, nv, page_size, float(scale), int(window) if window else 0,
-                int(chunk) if chunk else 0, float(softcap) if softcap else 0.0, _ptr(slopes), splits, _ptr(ws), int(meta.max_kv_len), self._s()))
+                int(chunk) if chunk else 0, float(softcap) if softcap else 0.0, _ptr(slopes), _ptr(sinks), splits, _ptr(ws), int(meta.max_kv_len), self._s()))
             return
         self._check(self.lib.lev_attention_values(
             _ptr(q), _rows(q, "attention_values: q"), _ptr(out), _ptr(k_pages), _ptr(v_pages), _ptr(meta.positions), _ptr(meta.token_seq),
             _ptr(block_tables), block_tables.shape[1], T, n_heads, n_kv_heads, head_dim, value_dim, nv, page_size, float(scale),
-            int(window) if window else 0, int(chunk) if chunk else 0, float(softcap) if softcap else 0.0, _ptr(slopes), _DT[dt], self._s()))
+            int(window) if window else 0, int(chunk) if chunk else 0, float(softcap) if softcap else 0.0, _ptr(slopes), _ptr(sinks), _DT[dt], self._s()))
 
     @staticmethod
     def mfma_attention_values_supports(head_dim: int, value_dim: int) -> bool:
@@ -738,6 +758,132 @@ class HipKernels:
             _ptr(u), _rows(u, "gated_recurrence: u"), _ptr(gates), _rows(gates, "gated_recurrence: gates"), _ptr(y), _rows(y, "gated_recurrence: y"),
             _ptr(x), _rows(x, "gated_recurrence: x"), _ptr(decay), _ptr(state), _ptr(token_slots), _ptr(out), _rows(out, "gated_recurrence: out"),
             T, C, state.shape[1], C // n_blocks, float(out_scale), _DT[dt], self._s()))
+
+    # ---- norms in groups around gated sublayers ------------------------------------------------
+    def group_norm_step(self, x, *, groups: int, eps: float, y=None, gate=None, post_weight=None, mult: float = 1.0, weight=None, h_out=None,
+                        rows=None, defer: bool = False, pending: Optional[PendingGatedNorm] = None) -> Optional[PendingGatedNorm]:
+        """One pass over the rows of the residual stream ``x`` (float32 ``[T, D]``) with ``gn(v, w)`` = ``v`` split into ``groups``
+        equal consecutive parts, each divided by its own ``sqrt(mean(part^2) + eps)``, times ``w``. In this order, whatever is
+        given: the write of a sublayer's result, ``x <- x + mult * gn(y * sigmoid(gate), post_weight)`` (``y`` float32 ``[T, D]``;
+        ``gate`` ``[T, D]`` float32 or compute dtype, rows may be strided, None: no gate); the read ``h_out = gn(x, weight)``
+        (compute dtype or float32). ``rows``: only these rows, into ``h_out [len(rows), D]``; ``x`` is not stored then.
+        ``defer``: nothing is launched; the write comes back as a ``PendingGatedNorm`` for the next call (``pending=``) or
+        ``finish``. ``pending``: the write of an earlier call, done in this pass."""
+        if pending is not None:
+            _req(pending.out is x and y is None and pending.groups == groups and pending.eps == eps, "group norm: the unfinished sublayer belongs to another tensor or norm")
+            y, gate, post_weight, mult = pending.y, pending.gate, pending.post_weight, pending.mult
+        if defer:
+            return PendingGatedNorm(x, y, gate, post_weight, float(mult), int(groups), float(eps))
+        _dev(x, y, gate, post_weight, weight, h_out, rows)
+        _req(x.dim() == 2 and x.dtype == torch.float32 and x.is_contiguous(), "group norm: x must be contiguous float32 [T, D]")
+        T, D = x.shape
+        _req(y is None or (y.dtype == torch.float32 and tuple(y.shape) == (T, D) and y.is_contiguous() and post_weight is not None),
+             "group norm: a sublayer's result must be contiguous float32 [T, D] and have a norm weight")
+        for name, w in (("post_weight", post_weight), ("weight", weight)):
+            _req(w is None or (w.dtype == torch.float32 and w.numel() == D and w.is_contiguous()), f"group norm: {name} must be float32 [D]")
+        gs, gdt = 0, torch.float32
+        if gate is not None:
+            _req(y is not None and gate.dtype in _DT and tuple(gate.shape) == (T, D), "group norm: the gate must be [T, D]")
+            gs, gdt = _rows(gate, "group norm: gate"), gate.dtype
+        n, odt = T, torch.float32
+        if rows is not None:
+            _req(rows.dtype == torch.int32 and rows.is_contiguous() and h_out is not None, "group norm: rows must be int32 and need an output")
+            n = rows.numel()
+        if h_out is not None:
+            _req(weight is not None and h_out.dtype in _DT and h_out.is_contiguous() and tuple(h_out.shape) == (n, D), "group norm: bad normalised output")
+            odt = h_out.dtype
+        self._check(self.lib.lev_group_norm_step(_ptr(x), _ptr(y), _ptr(gate), gs, _DT[gdt], _ptr(post_weight), float(mult), _ptr(weight), _ptr(h_out),
+                                                 _DT[odt], _ptr(rows), n, D, int(groups), float(eps), self._s()))
+        return None
+
+    # ---- rotation, "rotate half" layout --------------------------------------------------------
+    def rotary_half(self, x, n_heads: int, head_stride: int, offset: int, freqs, positions) -> None:
+        """In place on ``x`` ``[T, >= n_heads*head_stride]``: within each head of ``head_stride`` columns, the vector that starts at
+        column ``offset`` has its dimension i < len(freqs) paired with dimension i + len(freqs), and the pair turns by
+        ``positions[t] * freqs[i]``; every other column stays. 32-bit angles."""
+        _dev(x, freqs, positions)
+        T = x.shape[0]
+        _req(x.dim() == 2 and x.dtype in _DT and x.shape[1] >= n_heads * head_stride, "rotary: x must be [T, heads*head_stride]")
+        _req(freqs.dtype == torch.float32 and freqs.is_contiguous() and offset >= 0 and offset + 2 * freqs.numel() <= head_stride,
+             "rotary: float32 frequencies, and the rotated vector must fit the head")
+        _req(positions.dtype == torch.int32 and positions.numel() == T, "rotary: one int32 position per token")
+        self._check(self.lib.lev_rotary_half(_ptr(x), _rows(x, "rotary: x"), int(n_heads), int(head_stride), int(offset), freqs.numel(), _ptr(freqs),
+                                             _ptr(positions), T, _DT[x.dtype], self._s()))
+
+    # ---- a matrix state per head with decay and removal (generalized delta rule) ----------------
+    def delta_rule(self, r, k, v, a_pre, g, w_pre, norm_weight, state, token_slots, out, n_heads: int, head_dim: int, norm_eps: float,
+                   key_eps: float, sharpness: float) -> None:
+        """Per head, along each request's tokens, in 32-bit: ``u = k / sqrt(sum(k^2) + key_eps)``, ``w = exp(-sharpness *
+        sigmoid(w_pre))``, ``a = sigmoid(a_pre)``, ``S <- diag(w) S - (a * u)(u^T S) + k v^T`` (both terms read the old ``S``),
+        ``o = S^T r``, ``out = o / sqrt(mean(o^2) + norm_eps) * norm_weight * sigmoid(g)``. ``r, k, v, a_pre, g``: ``[T, H*d]``
+        views of one row stride in the compute dtype; ``w_pre`` float32 ``[T, H*d]``; ``state`` float32 ``[slots, H, d, d]``
+        (key channel, value channel), read and stored; ``token_slots`` int32 ``[T]`` (-1: a token of nobody, zeros)."""
+        _dev(r, k, v, a_pre, g, w_pre, norm_weight, state, token_slots, out)
+        T, C = r.shape
+        dt = r.dtype
+        _req(C == n_heads * head_dim and dt in _DT, "delta_rule: r must be [T, heads*head_dim] of a compute dtype")
+        stride = _rows(r, "delta_rule: r")
+        for name, t in (("k", k), ("v", v), ("a_pre", a_pre), ("g", g)):
+            _req(t.dtype == dt and tuple(t.shape) == (T, C) and _rows(t, f"delta_rule: {name}") == stride, f"delta_rule: {name} must be [T, heads*head_dim] with r's dtype and row stride")
+        _req(w_pre.dtype == torch.float32 and tuple(w_pre.shape) == (T, C), "delta_rule: w_pre must be float32 [T, heads*head_dim]")
+        _req(norm_weight.dtype == torch.float32 and norm_weight.numel() == C and norm_weight.is_contiguous(), "delta_rule: the norm's weight must be float32 [heads*head_dim]")
+        _req(state.dtype == torch.float32 and state.is_contiguous() and tuple(state.shape[1:]) == (n_heads, head_dim, head_dim), "delta_rule: state must be float32 [slots, heads, d, d]")
+        _req(token_slots.dtype == torch.int32 and token_slots.numel() == T, "delta_rule: one int32 slot per token")
+        _req(out.dtype == dt and tuple(out.shape) == (T, C), "delta_rule: out must be [T, heads*head_dim] of the compute dtype")
+        self._check(self.lib.lev_delta_rule(_ptr(r), _ptr(k), _ptr(v), _ptr(a_pre), _ptr(g), stride, _ptr(w_pre), _rows(w_pre, "delta_rule: w_pre"),
+                                            _ptr(norm_weight), _ptr(state), _ptr(token_slots), _ptr(out), _rows(out, "delta_rule: out"), T, n_heads,
+                                            head_dim, float(norm_eps), float(key_eps), float(sharpness), _DT[dt], self._s()))
+
+    # ---- mixture of experts --------------------------------------------------------------------
+    def moe_route(self, z, correction, chosen, weights, *, n_groups: int = 1, keep: int = 1, group_top: int = 2, renormalize: bool = False) -> None:
+        """Per token: ``s = sigmoid(z)`` (``z`` float32 ``[T, E]``); the choice goes by ``s + correction``; only experts of the
+        ``keep`` groups (of ``n_groups`` equal groups of neighbours) whose ``group_top`` largest choice scores sum highest can be
+        chosen; ``chosen`` int32 ``[T, top]`` the winners in the order of falling choice score (ties: lower index first),
+        ``weights`` float32 ``[T, top]`` their ``s`` (divided by their sum with ``renormalize``)."""
+        _dev(z, correction, chosen, weights)
+        T, E = z.shape
+        top = chosen.shape[1]
+        _req(z.dtype == torch.float32 and chosen.dtype == torch.int32 and weights.dtype == torch.float32, "experts: logits and weights float32, choices int32")
+        _req(tuple(chosen.shape) == tuple(weights.shape) == (T, top) and chosen.is_contiguous() and weights.is_contiguous(), "experts: choices and weights must be [T, top]")
+        _req(correction is None or (correction.dtype == torch.float32 and correction.numel() == E and correction.is_contiguous()), "experts: the correction must be float32 [E]")
+        self._check(self.lib.lev_moe_route(_ptr(z), _rows(z, "experts: z"), _ptr(correction), T, E, int(n_groups), int(keep), int(group_top), top,
+                                           int(renormalize), _ptr(chosen), _ptr(weights), self._s()))
+
+    def moe_max_tiles(self, pairs: int, n_experts: int) -> int:
+        return int(self.lib.lev_moe_max_tiles(int(pairs), int(n_experts)))
+
+    def moe_sort(self, chosen, n_experts: int, sorted_pairs, pos_of, tiles, meta) -> None:
+        """The (token, choice) pairs of ``chosen`` ordered by expert: ``sorted_pairs[pos]`` the pair at place ``pos``, ``pos_of`` its
+        inverse, ``tiles`` int32 ``[max_tiles, 3]`` (expert, first place, rows) covering every expert's stretch, ``meta[0]`` their
+        number. Everything stays on the device."""
+        _dev(chosen, sorted_pairs, pos_of, tiles, meta)
+        P = chosen.numel()
+        for t in (chosen, sorted_pairs, pos_of, tiles, meta):
+            _req(t.dtype == torch.int32 and t.is_contiguous(), "experts: int32 tables")
+        _req(sorted_pairs.numel() >= P and pos_of.numel() >= P and tiles.numel() >= 3 * self.moe_max_tiles(P, n_experts) and meta.numel() >= 1, "experts: tables too small")
+        self._check(self.lib.lev_moe_sort(_ptr(chosen), P, int(n_experts), _ptr(sorted_pairs), _ptr(pos_of), _ptr(tiles), _ptr(meta), self._s()))
+
+    def moe_linear(self, a, w, out, tiles, meta, sorted_pairs, *, top: int, gather: bool, glu: bool = False, activation: str = "none") -> None:
+        """For every tile of ``moe_sort``: ``out[pos] = w[expert] a[row(pos)]``, ``row(pos)`` the pair's token (``gather``) or
+        ``pos`` itself. ``w`` ``[E, N, K]``; with ``glu`` N = 2F, gate rows then up rows, and ``out[pos][f] = act(gate_f) * up_f``."""
+        _dev(a, w, out, tiles, meta, sorted_pairs)
+        _req(w.dim() == 3 and w.is_contiguous() and w.dtype in _DT and a.dtype == w.dtype and a.dim() == 2 and a.shape[1] == w.shape[2], "experts: a [rows, K], w [E, N, K] of one dtype")
+        E, N, K = w.shape
+        F_ = N // 2 if glu else N
+        _req(out.dim() == 2 and out.shape[1] == F_ and out.dtype in _DT and (a.dtype == torch.bfloat16 or out.dtype == torch.float32), "experts: bad output")
+        max_tiles = tiles.numel() // 3
+        self._check(self.lib.lev_moe_linear(_ptr(a), _rows(a, "experts: a"), _ptr(w), _ptr(out), _rows(out, "experts: out"), _ptr(tiles), _ptr(meta),
+                                            _ptr(sorted_pairs), max_tiles, int(top), int(gather), K, N, int(glu), ACTIVATIONS[activation], _DT[a.dtype],
+                                            _DT[out.dtype], int(self.use_mfma), self._s()))
+
+    def moe_combine(self, expert_out, pos_of, weights, y, accumulate: bool = False) -> None:
+        """``y[t] = sum_c weights[t, c] * expert_out[pos_of[t, c]]``, c in order, float32; ``accumulate``: added to what ``y`` holds."""
+        _dev(expert_out, pos_of, weights, y)
+        T, D = y.shape
+        top = weights.shape[1]
+        _req(expert_out.dtype == y.dtype == weights.dtype == torch.float32 and expert_out.is_contiguous() and y.is_contiguous() and weights.is_contiguous()
+             and expert_out.shape[1] == D and expert_out.shape[0] >= T * top and pos_of.dtype == torch.int32 and pos_of.numel() >= T * top, "experts: bad arguments of the weighted sum")
+        self._check(self.lib.lev_moe_combine(_ptr(expert_out), _ptr(pos_of), _ptr(weights), _ptr(y), T, D, top, int(accumulate), self._s()))
 
     # ---- attention -------------------------------------------------------------------------
     def paged_attention(self, q, out, k_pages, v_pages, meta, *, n_heads: int, n_kv_heads: int, head_dim: int,

@@ -1,6 +1,6 @@
 """Parts that layers are put together from. Importing the package registers the built-in kinds."""
-from . import (attention, block, embedding, feed_forward, head, hyper_connections, latent_attention, norm, parallel_mixers, position,  # noqa: F401
-               recurrent, stream_mix, talking_attention)
+from . import (attention, block, delta_rule, embedding, feed_forward, gated_block, head, hyper_connections, latent_attention, moe, norm,  # noqa: F401
+               parallel_mixers, position, recurrent, stream_mix, talking_attention)
 from .base import (AttentionMeta, Block, BuildEnv, CacheUnitView, Embedding, FeedForward, GroupView, Head, Mixer, Norm, Part,
                    PositionEncoding, StepContext, StreamMix)
 from .decoder import DecoderLm

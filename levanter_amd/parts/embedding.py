@@ -30,7 +30,8 @@ def tensors_of_nested(param: str, tensors: Dict[str, torch.Tensor]) -> Dict[str,
 @EMBEDDINGS.register("token_embedding")
 class TokenEmbedding(Embedding):
     """params: ``vocab_size``, ``dim``, ``position`` (the description of a position encoding, or None), ``scale`` (a
-    multiplier of the embedding's output, 1 by default); tensor ``table``."""
+    multiplier of the embedding's output, 1 by default), ``norm`` (the description of a norm that the residual stream's first
+    value goes through, or None; its class takes ``out_dtype`` and gives float32); tensor ``table``."""
 
     def __init__(self, spec: PartSpec, tensors: Dict[str, torch.Tensor], env: BuildEnv):
         super().__init__(spec, tensors, env)
@@ -42,10 +43,14 @@ class TokenEmbedding(Embedding):
         self.position = None
         if pos_spec is not None:
             self.position = part_class(pos_spec.kind, pos_spec.family or "position")(pos_spec, tensors_of_nested("position", tensors), env)
+        norm_spec: Optional[PartSpec] = spec.params.get("norm")
+        self.norm = None
+        if norm_spec is not None:
+            self.norm = part_class(norm_spec.kind, norm_spec.family or "norm")(norm_spec, tensors_of_nested("norm", tensors), env)
 
     @property
     def graph_safe(self) -> bool:
-        return self.position is None or bool(self.position.graph_safe)
+        return (self.position is None or bool(self.position.graph_safe)) and (self.norm is None or bool(self.norm.graph_safe))
 
     @property
     def max_positions(self) -> Optional[int]:
@@ -58,4 +63,6 @@ class TokenEmbedding(Embedding):
             ctx.kernels.embed(ctx.tokens, ctx.attention.positions, self.table, pos_table, x)
         else:
             ctx.kernels.embed(ctx.tokens, ctx.attention.positions, self.table, pos_table, x, scale=self.scale)
+        if self.norm is not None:
+            x = self.norm(x, ctx, out_dtype=torch.float32)
         return x

@@ -1,0 +1,93 @@
+"""A feed-forward made of many small experts of which every token uses a few (a mixture of experts).
+
+With h the feed-forward's input and E experts: router logits z = W_router h (32-bit sums), scores s = sigmoid(z). The choice
+goes by s + correction (a vector that only steers the choice); the experts form ``n_groups`` equal groups of neighbours, a
+group's score is the sum of its ``group_top`` largest choice scores, and only experts of the ``keep`` best groups can be chosen
+(the others count as minus infinity). The ``top`` experts with the largest choice scores run; the result is the sum of their
+outputs weighted by their s (divided by the sum of the chosen s with ``renormalize``). An expert is
+W_down (act(W_gate h) * (W_up h)) without biases.
+
+Nothing of the routing goes to the host: a kernel orders the step's (token, choice) pairs by expert and cuts every expert's
+stretch into row tiles, and the two products run over the tiles with a grid sized for the worst case (workgroups beyond the
+tiles that exist return at once), so the launches depend on the number of tokens alone and a step can be replayed from a
+HIP graph. Experts whose inner width is no multiple of 8 carry zeros behind it.
+"""
+from __future__ import annotations
+
+from typing import Dict
+
+import torch
+
+from levanter_amd.kernels.library import ACTIVATIONS
+from .base import BuildEnv, FeedForward, StepContext
+from .linear import Linear
+from .registry import FEED_FORWARDS
+from .spec import PartSpec
+
+
+@FEED_FORWARDS.register("routed_experts")
+class RoutedExperts(FeedForward):
+    """params: ``dim``, ``inner_dim``, ``n_experts``, ``top``, ``n_groups`` (1), ``keep`` (1), ``group_top`` (2), ``activation``
+    ("silu"), ``renormalize`` (False), ``correction`` (True: the tensor exists). Tensors: ``router.weight`` ``[E, dim]``,
+    ``correction`` ``[E]``, and per expert e ``experts.<e>.gate.weight``, ``experts.<e>.up.weight`` ``[inner, dim]``,
+    ``experts.<e>.down.weight`` ``[dim, inner]``."""
+
+    graph_safe = True
+
+    def __init__(self, spec: PartSpec, tensors: Dict[str, torch.Tensor], env: BuildEnv):
+        super().__init__(spec, tensors, env)
+        p = spec.params
+        self.dim, self.inner, self.n_experts, self.top = int(p["dim"]), int(p["inner_dim"]), int(p["n_experts"]), int(p["top"])
+        self.n_groups, self.keep, self.group_top = int(p.get("n_groups", 1)), int(p.get("keep", 1)), int(p.get("group_top", 2))
+        self.activation = p.get("activation", "silu")
+        self.renormalize = bool(p.get("renormalize", False))
+        if self.activation not in ACTIVATIONS:
+            raise ValueError(f"routed_experts: unknown activation {self.activation!r}")
+        E, D, F = self.n_experts, self.dim, self.inner
+        if E % self.n_groups or not 0 < self.keep <= self.n_groups or not 0 < self.top <= self.keep * (E // self.n_groups):
+            raise ValueError(f"routed_experts: {E} experts in {self.n_groups} groups, {self.keep} kept, {self.top} used")
+        Fp = self.inner_padded = (F + 7) // 8 * 8
+
+        def f32(name, shape):
+            t = tensors[name].to(torch.float32).cpu()
+            if tuple(t.shape) != tuple(shape):
+                raise ValueError(f"routed_experts: {name} must be {list(shape)}, got {list(t.shape)}")
+            return t
+
+        self.router = Linear(f32("router.weight", (E, D)), None, "out_in", env)
+        self.correction = f32("correction", (E,)).to(env.device).contiguous() if p.get("correction", True) else None
+        # [E, gate rows then up rows, dim] and [E, dim, inner]
+        w_in = torch.zeros(E, 2 * Fp, D)
+        w_down = torch.zeros(E, D, Fp)
+        for e in range(E):
+            w_in[e, :F] = f32(f"experts.{e}.gate.weight", (F, D))
+            w_in[e, Fp:Fp + F] = f32(f"experts.{e}.up.weight", (F, D))
+            w_down[e, :, :F] = f32(f"experts.{e}.down.weight", (D, F))
+        self.w_in = w_in.to(env.device, env.dtype).contiguous()
+        self.w_down = w_down.to(env.device, env.dtype).contiguous()
+
+    def forward(self, h: torch.Tensor, x: torch.Tensor, ctx: StepContext) -> None:
+        self._run(h, x, ctx, True)
+
+    def compute(self, h: torch.Tensor, y: torch.Tensor, ctx: StepContext) -> None:
+        self._run(h, y, ctx, False)
+
+    def _run(self, h: torch.Tensor, y: torch.Tensor, ctx: StepContext, accumulate: bool) -> None:
+        K = ctx.kernels
+        T, E, top = h.shape[0], self.n_experts, self.top
+        dev = h.device
+        z = self.router(h, ctx, out_dtype=torch.float32)
+        if accumulate:
+            ctx.settle()  # the sum below reads the residual stream itself
+        chosen = torch.empty((T, top), dtype=torch.int32, device=dev)
+        weights = torch.empty((T, top), dtype=torch.float32, device=dev)
+        K.moe_route(z, self.correction, chosen, weights, n_groups=self.n_groups, keep=self.keep, group_top=self.group_top, renormalize=self.renormalize)
+        P = T * top
+        tables = torch.empty(2 * P + 3 * K.moe_max_tiles(P, E) + 1, dtype=torch.int32, device=dev)
+        sorted_pairs, pos_of, meta, tiles = tables[:P], tables[P:2 * P], tables[2 * P:2 * P + 1], tables[2 * P + 1:]
+        K.moe_sort(chosen, E, sorted_pairs, pos_of, tiles, meta)
+        inner = ctx.empty(P, self.inner_padded)
+        K.moe_linear(h, self.w_in, inner, tiles, meta, sorted_pairs, top=top, gather=True, glu=True, activation=self.activation)
+        expert_out = ctx.empty(P, self.dim, torch.float32)
+        K.moe_linear(inner, self.w_down, expert_out, tiles, meta, sorted_pairs, top=top, gather=False)
+        K.moe_combine(expert_out, pos_of, weights, y, accumulate=accumulate)

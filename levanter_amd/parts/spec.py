@@ -22,6 +22,7 @@ class TensorSpec:
 
     name: str
     shape: Tuple[int, ...]
+    """A dimension of -1 is a size that only the checkpoint gives (any size fits; random weights cannot be drawn for it)."""
     kind: str = "float"  # "float": a real-valued tensor; "int": an integer table, kept as int32
     init: str = "normal"
     """Random-weights mode: "normal" = N(0, std); "one_plus_normal" = 1 + N(0, std); "eye_plus_normal" = identity + N(0, std)

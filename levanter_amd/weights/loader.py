@@ -69,7 +69,7 @@ def load_tensors(model_dir: str, spec: ModelSpec, device: str | torch.device = "
                 continue
             f, key = where[n]
             dtype, shape = f.info(key)
-            if tuple(shape) != tuple(ts.shape):
+            if len(shape) != len(ts.shape) or any(want != -1 and have != want for have, want in zip(shape, ts.shape)):  # -1: any size
                 wrong_shape.append(f"{n}: file has {list(shape)}, the configuration needs {list(ts.shape)}")
             is_float = dtype.is_floating_point
             if (ts.kind == "float") != is_float:

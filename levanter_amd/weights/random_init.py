@@ -25,6 +25,8 @@ def random_tensors(spec: ModelSpec, seed: int, dtype: torch.dtype = torch.float3
     out: Dict[str, torch.Tensor] = {}
     dev = torch.device(device)
     for name, ts in spec.all_tensors().items():
+        if any(d < 0 for d in ts.shape):
+            raise ValueError(f"tensor {name}: a size of it comes from a checkpoint alone ({list(ts.shape)}); the configuration must give it before weights can be drawn")
         g = torch.Generator(device=dev)
         g.manual_seed((int(seed) * 1000003 + zlib.crc32(name.encode())) % (2**63 - 1))
         if ts.kind == "int":

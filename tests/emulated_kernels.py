@@ -83,7 +83,7 @@ class EmulatedKernels:
 
     # ---- norm
     def norm(self, x, weight, bias, eps, out, rows=None, rms=False, pending=None) -> None:
-        if pending is not None:  # the only thing this stand-in leaves unfinished: a write into several residual streams
+        if pending is not None:  # what this stand-in leaves unfinished: a write into several residual streams, a gated sublayer
             self.finish(pending)
         src = x if rows is None else x[rows.long()]
         if rms:
@@ -95,6 +95,9 @@ class EmulatedKernels:
         out.copy_(y.to(out.dtype))
 
     def finish(self, pending) -> None:
+        if hasattr(pending, "post_weight"):
+            self.group_norm_step(pending.out, groups=pending.groups, eps=pending.eps, pending=pending)
+            return
         self.streams_step(pending.streams, y=pending.y, mix=pending.mix, w_out=pending.w_out, x_out=pending.out)  # a product is never left unfinished here
 
     # ---- several residual streams
@@ -186,6 +189,125 @@ class EmulatedKernels:
             hist = torch.cat([state[slot, :K - 1], x[t:t + n].float()], 0)
             state[slot, :K - 1] = hist[hist.shape[0] - (K - 1):]
             t += n
+
+    # ---- norms in groups around gated sublayers
+    @staticmethod
+    def _group_norm(v, w, groups, eps):
+        T, D = v.shape
+        parts = v.view(T, groups, D // groups)
+        return (parts / torch.sqrt((parts * parts).mean(-1, keepdim=True) + eps)).reshape(T, D) * w
+
+    def group_norm_step(self, x, *, groups, eps, y=None, gate=None, post_weight=None, mult=1.0, weight=None, h_out=None, rows=None, defer=False,
+                        pending=None):
+        if pending is not None:
+            assert pending.out is x and y is None
+            y, gate, post_weight, mult = pending.y, pending.gate, pending.post_weight, pending.mult
+        if defer:
+            from types import SimpleNamespace
+
+            return SimpleNamespace(out=x, y=y, gate=gate, post_weight=post_weight, mult=float(mult), groups=int(groups), eps=float(eps))
+        cur = x
+        if y is not None:
+            z = y if gate is None else y * torch.sigmoid(gate.float())
+            cur = x + mult * self._group_norm(z, post_weight, groups, eps)
+            if rows is None:
+                x.copy_(cur)
+        if h_out is not None:
+            src = cur if rows is None else cur[rows.long()]
+            h_out.copy_(self._group_norm(src, weight, groups, eps).to(h_out.dtype))
+        return None
+
+    # ---- rotation, rotate-half layout
+    def rotary_half(self, x, n_heads, head_stride, offset, freqs, positions) -> None:
+        n = freqs.numel()
+        if n == 0:
+            return
+        a = positions.float()[:, None] * freqs[None, :]
+        cos, sin = torch.cos(a)[:, None, :], torch.sin(a)[:, None, :]
+        v = x[:, :n_heads * head_stride].view(x.shape[0], n_heads, head_stride)
+        lo, hi = v[:, :, offset:offset + n].float().clone(), v[:, :, offset + n:offset + 2 * n].float().clone()
+        v[:, :, offset:offset + n] = (lo * cos - hi * sin).to(x.dtype)
+        v[:, :, offset + n:offset + 2 * n] = (hi * cos + lo * sin).to(x.dtype)
+
+    # ---- generalized delta rule
+    def delta_rule(self, r, k, v, a_pre, g, w_pre, norm_weight, state, token_slots, out, n_heads, head_dim, norm_eps, key_eps, sharpness) -> None:
+        T, H, d = r.shape[0], n_heads, head_dim
+        nw = norm_weight.view(H, d)
+        for t in range(T):
+            slot = int(token_slots[t])
+            if slot < 0:
+                out[t] = 0
+                continue
+            kf, rf, vf = (z[t].float().view(H, d) for z in (k, r, v))
+            u = kf / torch.sqrt((kf * kf).sum(-1, keepdim=True) + key_eps)
+            w = torch.exp(-sharpness * torch.sigmoid(w_pre[t].float().view(H, d)))
+            a = torch.sigmoid(a_pre[t].float().view(H, d))
+            S = state[slot]
+            uS = torch.einsum("hi,hij->hj", u, S)
+            S = w[:, :, None] * S - (a * u)[:, :, None] * uS[:, None, :] + kf[:, :, None] * vf[:, None, :]
+            state[slot] = S
+            o = torch.einsum("hij,hi->hj", S, rf)
+            o = o / torch.sqrt((o * o).mean(-1, keepdim=True) + norm_eps) * nw * torch.sigmoid(g[t].float().view(H, d))
+            out[t] = o.reshape(-1).to(out.dtype)
+
+    # ---- mixture of experts
+    def moe_route(self, z, correction, chosen, weights, *, n_groups=1, keep=1, group_top=2, renormalize=False) -> None:
+        T, E = z.shape
+        top = chosen.shape[1]
+        s = torch.sigmoid(z.float())
+        c = s if correction is None else s + correction
+        per = E // n_groups
+        for t in range(T):
+            ct = c[t].clone()
+            if n_groups > 1:
+                scores = [sum(sorted(ct[g * per:(g + 1) * per].tolist(), reverse=True)[:group_top]) for g in range(n_groups)]
+                order = sorted(range(n_groups), key=lambda g: (-scores[g], g))
+                for g in order[keep:]:
+                    ct[g * per:(g + 1) * per] = -math.inf
+            order = sorted(range(E), key=lambda e: (-float(ct[e]), e))[:top]
+            chosen[t] = torch.tensor(order, dtype=torch.int32)
+            wt = s[t][order]
+            weights[t] = wt / wt.sum() if renormalize else wt
+
+    TILE_ROWS = 16
+
+    def moe_max_tiles(self, pairs, n_experts) -> int:
+        return pairs // self.TILE_ROWS + n_experts + 1
+
+    def moe_sort(self, chosen, n_experts, sorted_pairs, pos_of, tiles, meta) -> None:
+        flat = chosen.reshape(-1).long()
+        order = torch.sort(flat, stable=True).indices
+        P = flat.numel()
+        sorted_pairs[:P] = order.to(torch.int32)
+        pos_of[order] = torch.arange(P, dtype=torch.int32)
+        tl = tiles.view(-1, 3)
+        n, at = 0, 0
+        for e in range(n_experts):
+            count = int((flat == e).sum())
+            for i in range(0, count, self.TILE_ROWS):
+                tl[n] = torch.tensor([e, at + i, min(self.TILE_ROWS, count - i)], dtype=torch.int32)
+                n += 1
+            at += count
+        meta[0] = n
+
+    def moe_linear(self, a, w, out, tiles, meta, sorted_pairs, *, top, gather, glu=False, activation="none") -> None:
+        tl = tiles.view(-1, 3)
+        F_ = out.shape[1]
+        for i in range(int(meta[0])):
+            e, first, n = (int(v) for v in tl[i])
+            pos = torch.arange(first, first + n)
+            src = (sorted_pairs[pos].long() // top) if gather else pos
+            y = a[src].float() @ w[e].float().t()
+            if glu:
+                y = _act(activation)(y[:, :F_]) * y[:, F_:]
+            out[pos] = y.to(out.dtype)
+
+    def moe_combine(self, expert_out, pos_of, weights, y, accumulate=False) -> None:
+        T, top = weights.shape
+        acc = y.clone() if accumulate else torch.zeros_like(y)
+        for c in range(top):
+            acc = acc + weights[:, c:c + 1] * expert_out[pos_of.view(T, top)[:, c].long()]
+        y.copy_(acc)
 
     # ---- linear
     def linear(self, a, w, bias, out, activation="none", residual=None, may_leave_pending=False) -> None:
@@ -323,7 +445,7 @@ class EmulatedKernels:
         x.copy_(acc)
 
     def attention_values(self, q, out, k_pages, v_pages, meta, *, n_heads, n_kv_heads, head_dim, value_dim, all_value_heads, page_size,
-                         scale, window, block_tables, softcap=None, slopes=None, chunk=None) -> None:
+                         scale, window, block_tables, softcap=None, slopes=None, chunk=None, sinks=None) -> None:
         T = q.shape[0]
         g = n_heads // n_kv_heads
         o = out.view(T, n_heads, n_kv_heads if all_value_heads else 1, value_dim)
@@ -339,7 +461,10 @@ class EmulatedKernels:
                 s = softcap * torch.tanh(s / softcap)
             if slopes is not None:
                 s = s - slopes.float()[:, None] * (pos - torch.arange(lo, pos + 1)).float()[None, :]
-            p = torch.softmax(s, -1)
+            if sinks is not None:  # a score without a key and without a value in the denominator
+                p = torch.softmax(torch.cat([s, sinks.float()[:, None]], -1), -1)[:, :-1]
+            else:
+                p = torch.softmax(s, -1)
             if all_value_heads:
                 o[t] = torch.einsum("hn,cnd->hcd", p, vs.float())
             else:

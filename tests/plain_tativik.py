@@ -1,0 +1,201 @@
+"""Tativik, stated plainly: whole sequences in float64, one function per mechanism, no cache, no kernels, nothing shared
+with the package. ``weights`` maps checkpoint tensor names to float64 tensors, ``cfg`` is the raw config.json dict.
+
+Notation: x the residual stream ``[T, D]``, h a sublayer's input, positions count from 0.
+"""
+from __future__ import annotations
+
+import math
+from typing import Dict, List, Optional, Tuple
+
+import torch
+
+F64 = torch.float64
+
+
+# ---- norms ------------------------------------------------------------------------------------------------------
+def rms_norm(x: torch.Tensor, w: Optional[torch.Tensor], eps: float) -> torch.Tensor:
+    """x / sqrt(mean(x^2) + eps) over the last dimension, times w."""
+    y = x / torch.sqrt((x * x).mean(-1, keepdim=True) + eps)
+    return y if w is None else y * w
+
+
+def group_rms_norm(x: torch.Tensor, w: torch.Tensor, groups: int, eps: float) -> torch.Tensor:
+    """The last dimension in ``groups`` equal consecutive parts, each divided by its own root mean square; then times w."""
+    T, D = x.shape
+    parts = x.view(T, groups, D // groups)
+    return rms_norm(parts, None, eps).reshape(T, D) * w
+
+
+# ---- positions --------------------------------------------------------------------------------------------------
+def rotate_half(v: torch.Tensor, positions: torch.Tensor, dims: int, base: float) -> torch.Tensor:
+    """v ``[T, ..., n]``: dimension i < dims/2 is paired with i + dims/2 and the pair turned by p * base^(-2i/dims); dimensions
+    from ``dims`` on pass unchanged."""
+    half = dims // 2
+    out = v.clone()
+    if half == 0:
+        return out
+    f = torch.tensor([float(base) ** (-2.0 * i / dims) for i in range(half)], dtype=F64)
+    a = positions.to(F64)[:, None] * f[None, :]
+    shape = [v.shape[0]] + [1] * (v.dim() - 2) + [half]
+    cos, sin = torch.cos(a).view(shape), torch.sin(a).view(shape)
+    lo, hi = v[..., :half], v[..., half:dims]
+    out[..., :half] = lo * cos - hi * sin
+    out[..., half:dims] = hi * cos + lo * sin
+    return out
+
+
+def window_visible(T: int, size: Optional[int]) -> torch.Tensor:
+    """[T, T] bool: query i sees key j iff 0 <= i - j < size (no size: every j <= i)."""
+    i = torch.arange(T)[:, None]
+    j = torch.arange(T)[None, :]
+    ok = j <= i
+    if size is not None:
+        ok = ok & (i - j < size)
+    return ok
+
+
+def softmax_with_sink(scores: torch.Tensor, visible: torch.Tensor, sink: Optional[torch.Tensor]) -> torch.Tensor:
+    """scores ``[H, T, T]``; weights over the visible keys whose denominator also holds exp(sink_h), once per row."""
+    s = scores.masked_fill(~visible[None], -math.inf)
+    m = s.max(-1, keepdim=True).values
+    if sink is not None:
+        m = torch.maximum(m, sink.view(-1, 1, 1))
+    e = torch.exp(s - m)
+    den = e.sum(-1, keepdim=True)
+    if sink is not None:
+        den = den + torch.exp(sink.view(-1, 1, 1) - m)
+    return e / den
+
+
+# ---- latent attention ---------------------------------------------------------------------------------------------
+def latent_kv(h: torch.Tensor, w_dkv: torch.Tensor, norm_w: torch.Tensor, kv_rank: int, eps: float, rot_dims: int, base: float
+              ) -> Tuple[torch.Tensor, torch.Tensor]:
+    """What a layer caches: the normed latent ``[T, kv_rank]`` and the rotated key part ``[T, rot_dim]`` that all heads share."""
+    d = h @ w_dkv.T
+    c = rms_norm(d[:, :kv_rank], norm_w, eps)
+    k_rot = rotate_half(d[:, kv_rank:], torch.arange(h.shape[0]), rot_dims, base)
+    return c, k_rot
+
+
+def latent_attention(h: torch.Tensor, W: Dict[str, torch.Tensor], p: str, m: dict, eps: float,
+                     kv: Optional[Tuple[torch.Tensor, torch.Tensor]] = None) -> Tuple[torch.Tensor, Tuple[torch.Tensor, torch.Tensor]]:
+    """The mixer's output ``[T, D]`` and the (latent, rotated key part) it used: its own, or ``kv`` of the layer it borrows from."""
+    T = h.shape[0]
+    H, dk, dr, dv, R = m["heads"], m["dim"], m["rot_dim"], m["vdim"], m["kv_rank"]
+    rot = m.get("rot") or {}
+    rot_dims, base = int(rot.get("dims", 0)), float(rot.get("base", 10000.0))
+    cq = rms_norm(h @ W[f"{p}.dq"].T, W[f"{p}.dq.norm"], eps)
+    q = (cq @ W[f"{p}.uq"].T).view(T, H, dk + dr)
+    q_plain = q[..., :dk]
+    q_rot = rotate_half(q[..., dk:], torch.arange(T), rot_dims, base)
+    if kv is None:
+        kv = latent_kv(h, W[f"{p}.dkv"], W[f"{p}.dkv.norm"], R, eps, rot_dims, base)
+    c, k_rot = kv
+    k_plain = (c @ W[f"{p}.uk"].T).view(T, H, dk)
+    v = (c @ W[f"{p}.uv"].T).view(T, H, dv)
+    scores = (torch.einsum("ihd,jhd->hij", q_plain, k_plain) + torch.einsum("ihd,jd->hij", q_rot, k_rot)) * float(m["scale"])
+    size = (m.get("mask") or {}).get("size")
+    weights = softmax_with_sink(scores, window_visible(T, size), W.get(f"{p}.sink"))
+    o = torch.einsum("hij,jhd->ihd", weights, v)
+    o = o * torch.sigmoid(h @ W[f"{p}.g"].T)[:, :, None]
+    return o.reshape(T, H * dv) @ W[f"{p}.o"].T, kv
+
+
+# ---- generalized delta rule ---------------------------------------------------------------------------------------
+DECAY_SHARPNESS = math.exp(-0.5)
+UNIT_KEY_EPS = 1e-6
+
+
+def delta_rule_scan(r, k, v, w, a, state=None):
+    """Per head: S <- diag(w_t) S - (a_t * u_t)(u_t^T S) + k_t v_t^T with u = k / sqrt(sum(k^2) + 1e-6), both terms reading the old
+    S; o_t = S^T r_t. All ``[T, H, d]``; returns o ``[T, H, d]`` and the last state ``[H, d, d]`` (key channel, value channel)."""
+    T, H, d = k.shape
+    S = torch.zeros(H, d, d, dtype=F64) if state is None else state.clone()
+    u = k / torch.sqrt((k * k).sum(-1, keepdim=True) + UNIT_KEY_EPS)
+    out = torch.empty(T, H, d, dtype=F64)
+    for t in range(T):
+        uS = torch.einsum("hi,hij->hj", u[t], S)
+        S = w[t][:, :, None] * S - (a[t] * u[t])[:, :, None] * uS[:, None, :] + k[t][:, :, None] * v[t][:, None, :]
+        out[t] = torch.einsum("hij,hi->hj", S, r[t])
+    return out, S
+
+
+def general_delta(h: torch.Tensor, W: Dict[str, torch.Tensor], p: str, m: dict, eps: float) -> torch.Tensor:
+    T = h.shape[0]
+    H, d = m["heads"], m["dim"]
+    r, k, v = ((h @ W[f"{p}.{n}"].T).view(T, H, d) for n in ("r", "k", "v"))
+    w = torch.exp(-DECAY_SHARPNESS * torch.sigmoid(torch.tanh(h @ W[f"{p}.w1"].T) @ W[f"{p}.w2"].T + W[f"{p}.w0"])).view(T, H, d)
+    a = torch.sigmoid(h @ W[f"{p}.a"].T + W[f"{p}.a.b"]).view(T, H, d)
+    o, _ = delta_rule_scan(r, k, v, w, a)
+    o = rms_norm(o, None, eps).reshape(T, H * d) * W[f"{p}.norm"]
+    o = o * torch.sigmoid(h @ W[f"{p}.g"].T)
+    return o @ W[f"{p}.o"].T
+
+
+# ---- mixture of experts -------------------------------------------------------------------------------------------
+def route(z: torch.Tensor, correction: torch.Tensor, top: int, n_groups: int, keep: int) -> Tuple[torch.Tensor, torch.Tensor]:
+    """z ``[T, E]`` router logits. Returns the chosen experts ``[T, top]`` and their weights: s = sigmoid(z); the choice goes by
+    s + correction among the experts of the ``keep`` groups whose two largest choice scores sum highest; the weights are s."""
+    T, E = z.shape
+    s = torch.sigmoid(z)
+    choice = s + correction
+    per = E // n_groups
+    grouped = choice.view(T, n_groups, per)
+    group_score = grouped.topk(min(2, per), -1).values.sum(-1)
+    kept = group_score.topk(keep, -1).indices
+    allowed = torch.zeros(T, n_groups, dtype=torch.bool).scatter_(1, kept, True)
+    masked = choice.masked_fill(~allowed[:, :, None].expand(T, n_groups, per).reshape(T, E), -math.inf)
+    chosen = masked.topk(top, -1).indices
+    return chosen, s.gather(1, chosen)
+
+
+def expert(h: torch.Tensor, W: Dict[str, torch.Tensor], p: str) -> torch.Tensor:
+    g = h @ W[f"{p}.gate"].T
+    return ((g * torch.sigmoid(g)) * (h @ W[f"{p}.up"].T)) @ W[f"{p}.down"].T
+
+
+def moe(h: torch.Tensor, W: Dict[str, torch.Tensor], p: str, mlp: dict) -> torch.Tensor:
+    r = mlp["router"]
+    groups = r.get("groups") or {"count": 1, "keep": 1}
+    chosen, weights = route(h @ W[f"{p}.router"].T, W[f"{p}.correction"], r["top"], groups["count"], groups["keep"])
+    out = torch.zeros_like(h)
+    for t in range(h.shape[0]):
+        for e, wt in zip(chosen[t].tolist(), weights[t]):
+            out[t] += wt * expert(h[t:t + 1], W, f"{p}.e{e}")[0]
+    return out
+
+
+# ---- the model ----------------------------------------------------------------------------------------------------
+def forward(cfg: dict, W: Dict[str, torch.Tensor], tokens: List[int], return_layers: bool = False):
+    """Logits ``[T, vocab]`` of one whole sequence (and the residual stream after every layer)."""
+    eps, groups, mult = float(cfg["norm"]["eps"]), int(cfg["norm"]["groups"]), float(cfg["residual_mult"])
+
+    def norm(x, name):
+        return group_rms_norm(x, W[name], groups, eps)
+
+    x = norm(W["embed"][torch.tensor(tokens)], "embed.norm")
+    kept: Dict[int, Tuple[torch.Tensor, torch.Tensor]] = {}
+    after = []
+    for i, layer in enumerate(cfg["layers"]):
+        p, m = f"l{i}", layer["mixer"]
+        h = norm(x, f"{p}.norm1")
+        if layer["type"] == "latent_attention":
+            src = m.get("kv_from")
+            y, kv = latent_attention(h, W, f"{p}.mix", m, eps, None if src is None else kept[src])
+            if src is None:
+                kept[i] = kv
+        elif layer["type"] == "general_delta":
+            y = general_delta(h, W, f"{p}.mix", m, eps)
+        else:
+            raise ValueError(layer["type"])
+        y = y * torch.sigmoid(h @ W[f"{p}.rg1"].T + W[f"{p}.rg1.b"])
+        x = x + mult * norm(y, f"{p}.norm1b")
+        if layer.get("mlp") is not None:
+            h = norm(x, f"{p}.norm2")
+            y = moe(h, W, f"{p}.mlp", layer["mlp"])
+            y = y * torch.sigmoid(h @ W[f"{p}.rg2"].T + W[f"{p}.rg2.b"])
+            x = x + mult * norm(y, f"{p}.norm2b")
+        after.append(x)
+    logits = norm(x, "final.norm") @ W["head"].T
+    return (logits, torch.stack(after)) if return_layers else logits

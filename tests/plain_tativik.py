@@ -199,3 +199,119 @@ def forward(cfg: dict, W: Dict[str, torch.Tensor], tokens: List[int], return_lay
         after.append(x)
     logits = norm(x, "final.norm") @ W["head"].T
     return (logits, torch.stack(after)) if return_layers else logits
+
+
+def plain_logits(W: Dict[str, torch.Tensor], cfg: dict, tokens) -> torch.Tensor:
+    return forward(cfg, W, [int(t) for t in tokens])
+
+
+def plain_greedy(W: Dict[str, torch.Tensor], cfg: dict, prompt: List[int], n_new: int) -> List[int]:
+    toks = list(prompt)
+    for _ in range(n_new):
+        toks.append(int(torch.argmax(forward(cfg, W, toks)[-1])))
+    return toks[len(prompt):]
+
+
+# ---- small configurations and weights for the tests ---------------------------------------------------------------------
+def latent_layer(heads=4, dim=16, rot_dim=8, vdim=8, kv_rank=24, q_rank=16, window=None, rot_dims=None, base=10000.0, scale=None, kv_from=None,
+                 mlp="default") -> dict:
+    m = {"heads": heads, "dim": dim, "rot_dim": rot_dim, "vdim": vdim, "kv_rank": kv_rank, "q_rank": q_rank,
+         "scale": scale if scale is not None else 1.0 / math.sqrt(dim + rot_dim)}
+    if rot_dim:
+        m["rot"] = {"dims": rot_dim if rot_dims is None else rot_dims, "base": base}
+    if window is not None:
+        m["mask"] = {"size": window}
+    if kv_from is not None:
+        m["kv_from"] = kv_from
+    return {"type": "latent_attention", "mixer": m, "mlp": experts_mlp() if mlp == "default" else mlp}
+
+
+def delta_layer(heads=2, dim=16, decay_rank=8, mlp="default") -> dict:
+    return {"type": "general_delta", "mixer": {"heads": heads, "dim": dim, "decay_rank": decay_rank}, "mlp": experts_mlp() if mlp == "default" else mlp}
+
+
+def experts_mlp(ff=24, experts=8, top=2, groups=None) -> dict:
+    router = {"experts": experts, "top": top}
+    if groups is not None:
+        router["groups"] = {"count": groups[0], "keep": groups[1]}
+    return {"kind": "moe", "expert": {"ff": ff}, "router": router}
+
+
+def make_config(vocab=97, width=64, layers=None, eps=1e-5, groups=2, mult=0.7) -> dict:
+    return {"architecture": "Tativik", "vocab": vocab, "width": width, "norm": {"eps": eps, "groups": groups}, "residual_mult": mult, "layers": layers}
+
+
+def random_weights(cfg: dict, seed: int, dtype=F64) -> Dict[str, torch.Tensor]:
+    """Weights drawn so that every mechanism matters: scores of order one, sinks that take a visible share of the weight,
+    gates that are not saturated, decays and removal rates over their whole range, router scores whose order the correction
+    changes. Values are bfloat16 numbers (a file stores them exactly)."""
+    g = torch.Generator().manual_seed(seed)
+    D, V = cfg["width"], cfg["vocab"]
+
+    def rn(*shape, std=1.0):
+        return (torch.randn(*shape, generator=g) * std).to(torch.bfloat16).to(dtype)
+
+    W = {"embed": rn(V, D), "embed.norm": 1 + rn(D, std=0.2), "final.norm": 1 + rn(D, std=0.2), "head": rn(V, D, std=1 / math.sqrt(D))}
+    for i, L in enumerate(cfg["layers"]):
+        m, p = L["mixer"], f"l{i}."
+        for n in ("norm1", "norm1b"):
+            W[p + n] = 1 + rn(D, std=0.2)
+        W[p + "rg1"] = rn(D, D, std=1 / math.sqrt(D))
+        W[p + "rg1.b"] = rn(D, std=0.5)
+        if L["type"] == "latent_attention":
+            H, dk, dr, dv, R, Q = m["heads"], m["dim"], m["rot_dim"], m["vdim"], m["kv_rank"], m["q_rank"]
+            W[p + "mix.dq"] = rn(Q, D, std=1 / math.sqrt(D))
+            W[p + "mix.dq.norm"] = 1 + rn(Q, std=0.2)
+            W[p + "mix.uq"] = rn(H * (dk + dr), Q, std=1.5 / math.sqrt(Q))
+            if m.get("kv_from") is None:
+                W[p + "mix.dkv"] = rn(R + dr, D, std=1.5 / math.sqrt(D))
+                W[p + "mix.dkv.norm"] = 1 + rn(R, std=0.2)
+            W[p + "mix.uk"] = rn(H * dk, R, std=1.5 / math.sqrt(R))
+            W[p + "mix.uv"] = rn(H * dv, R, std=1 / math.sqrt(R))
+            W[p + "mix.sink"] = rn(H, std=1.5)
+            W[p + "mix.g"] = rn(H, D, std=1.5 / math.sqrt(D))
+            W[p + "mix.o"] = rn(D, H * dv, std=1 / math.sqrt(H * dv))
+        else:
+            H, d, rank = m["heads"], m["dim"], m["decay_rank"]
+            C = H * d
+            for n in ("r", "k", "v", "g", "a"):
+                W[p + f"mix.{n}"] = rn(C, D, std=1 / math.sqrt(D))
+            W[p + "mix.a.b"] = rn(C, std=1.0)
+            W[p + "mix.w1"] = rn(rank, D, std=1 / math.sqrt(D))
+            W[p + "mix.w2"] = rn(C, rank, std=2 / math.sqrt(rank))
+            W[p + "mix.w0"] = rn(C, std=1.5)
+            W[p + "mix.norm"] = 1 + rn(C, std=0.2)
+            W[p + "mix.o"] = rn(D, C, std=1 / math.sqrt(C))
+        mlp = L.get("mlp")
+        if mlp is not None:
+            F, E = mlp["expert"]["ff"], mlp["router"]["experts"]
+            for n in ("norm2", "norm2b"):
+                W[p + n] = 1 + rn(D, std=0.2)
+            W[p + "rg2"] = rn(D, D, std=1 / math.sqrt(D))
+            W[p + "rg2.b"] = rn(D, std=0.5)
+            W[p + "mlp.router"] = rn(E, D, std=1.5 / math.sqrt(D))
+            W[p + "mlp.correction"] = rn(E, std=0.3)
+            for e in range(E):
+                W[p + f"mlp.e{e}.gate"] = rn(F, D, std=1 / math.sqrt(D))
+                W[p + f"mlp.e{e}.up"] = rn(F, D, std=1 / math.sqrt(D))
+                W[p + f"mlp.e{e}.down"] = rn(D, F, std=1 / math.sqrt(F))
+    return W
+
+
+def write_folder(cfg: dict, W: Dict[str, torch.Tensor], path: str, dtype=torch.bfloat16) -> str:
+    """config.json and model.safetensors of these weights, through the safetensors package. The inner size of the decay's map
+    is left to the tensors: the written configuration does not name it."""
+    import copy
+    import json
+    import os
+
+    from safetensors.torch import save_file
+
+    os.makedirs(path, exist_ok=True)
+    out = copy.deepcopy(cfg)
+    for L in out["layers"]:
+        L["mixer"].pop("decay_rank", None)
+    with open(os.path.join(path, "config.json"), "w") as f:
+        json.dump(out, f)
+    save_file({k: v.to(dtype).contiguous() for k, v in W.items()}, os.path.join(path, "model.safetensors"))
+    return path

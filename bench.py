@@ -55,15 +55,16 @@ def main() -> int:
     ap.add_argument("--shape", default="7b", choices=["7b", "xl", "20b"],
                     help="layer sizes of the decode workload: 7b is the headline's; xl and 20b measure the same step at the other "
                          "sizes of the reference's configurations (use --no-points: the prefill point is 2,048 tokens)")
-    ap.add_argument("--workload", default="decode", choices=["decode", "xl_mix", "20b", "zederax", "nakurax"],
+    ap.add_argument("--workload", default="decode", choices=["decode", "xl_mix", "20b", "zederax", "nakurax", "tativik"],
                     help="decode: the workload described above. xl_mix / 20b: continuous-batching workloads at the gpt2_xl and gpt2_20b sizes "
                          "through InferenceEngine.generate; they print their own line. zederax: prefill and decode rates of Zederax "
                          "layers at a few sizes beside GPT-2 layers of the same width, heads and inner width; its own line. nakurax: the same for "
-                         "Nakurax layers (latent attention and attention beside a recurrence, in turn) beside Zederax and GPT-2 layers")
+                         "Nakurax layers (latent attention and attention beside a recurrence, in turn) beside Zederax and GPT-2 layers. tativik: Tativik "
+                         "layers (windowed latent attention with a rotated key part and a generalized delta rule, in turn, routed experts) beside Nakurax layers")
     ap.add_argument("--sizes", default="1k,2k,4k", help="with --workload zederax / nakurax: which of the sizes 1k, 2k, 4k to run")
     ap.add_argument("--batches", default="1,8,64", help="with --workload zederax: decode batch sizes to time ('' for none)")
     ap.add_argument("--no-prefill", action="store_true", help="with --workload zederax: skip the 2,048-token prompt")
-    ap.add_argument("--arch", default="both", choices=["both", "zederax", "gpt2", "nakurax"],
+    ap.add_argument("--arch", default="both", choices=["both", "zederax", "gpt2", "nakurax", "tativik"],
                     help="with --workload zederax / nakurax: one architecture only (for profiling)")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -75,7 +76,7 @@ def main() -> int:
     from levanter_amd.config import InferenceEngineConfig, LmConfig
     from levanter_amd.engine import InferenceEngine, Request
 
-    if args.workload in ("zederax", "nakurax"):
+    if args.workload in ("zederax", "nakurax", "tativik"):
         return zederax_workload(args)
     if args.workload != "decode":
         return serving_workload(args)
@@ -343,6 +344,24 @@ def nakurax_config(z):
             "streams": 4, "layers": layers}
 
 
+def tativik_config(z):
+    """Latent-attention layers (queries through a latent, a rotated key part of 32, a window, sinks, gates) and layers of the
+    generalized delta rule, in turn, every sublayer between two norms in two groups and behind a gate; the heads, head sizes and
+    layer count of the size, a latent of two key heads' size (at most 224, so that latent and rotated part fill a key of 256).
+    The feed-forward has 32 experts of a quarter of the size's inner width in 8 groups of which 4 are kept, 4 experts a token:
+    a token's experts hold as much as the size's dense feed-forward."""
+    import math
+
+    rot = 32
+    latent = {"heads": z["heads"], "dim": z["dim"], "rot_dim": rot, "vdim": z["vdim"], "kv_rank": min(224, 2 * z["dim"]), "q_rank": z["width"] // 2,
+              "scale": 1.0 / math.sqrt(z["dim"] + rot), "rot": {"dims": rot, "base": 500000.0}, "mask": {"size": z["window"]}}
+    delta = {"heads": z["width"] // z["dim"], "dim": z["dim"], "decay_rank": 64}
+    mlp = {"kind": "moe", "expert": {"ff": z["ff"] // 4}, "router": {"experts": 32, "top": 4, "groups": {"count": 8, "keep": 4}}}
+    layers = [{"type": "latent_attention" if i % 2 == 0 else "general_delta", "mixer": dict(latent if i % 2 == 0 else delta), "mlp": json.loads(json.dumps(mlp))}
+              for i in range(z["layers"])]
+    return {"architecture": "Tativik", "vocab": ZEDERAX_VOCAB, "width": z["width"], "norm": {"eps": 1e-6, "groups": 2}, "residual_mult": 0.7, "layers": layers}
+
+
 def zederax_workload(args) -> int:
     """Prefill (one 2,048-token prompt) and decode (batch 1, 8, 64 after 512-token prompts) through the engine, for Zederax
     (or, with --workload nakurax, Nakurax and Zederax) and for GPT-2 at equal sizes. One JSON line."""
@@ -414,11 +433,14 @@ def zederax_workload(args) -> int:
         archs = [("zederax", zederax_config(z)), ("gpt2", gpt2_config_like(z))]
         if args.workload == "nakurax":
             archs.insert(0, ("nakurax", nakurax_config(z)))
+        if args.workload == "tativik":  # beside the closest model: Nakurax's latent attention and recurrence
+            archs = [("tativik", tativik_config(z)), ("nakurax", nakurax_config(z))]
         for arch, raw in archs:
             if args.arch in ("both", arch):
                 print(f"[bench] {arch} at size {name} ...", file=sys.stderr, flush=True)
                 results[name][arch] = measure(raw)
-    print(json.dumps({"metric": f"prefill and decode tok/s of {args.workload.capitalize()} layers beside {'Zederax and ' if args.workload == 'nakurax' else ''}GPT-2 layers of equal width, heads and inner width",
+    print(json.dumps({"metric": (f"prefill and decode tok/s of Tativik layers beside Nakurax layers of equal width, heads and (per token) inner width" if args.workload == "tativik" else
+                                 f"prefill and decode tok/s of {args.workload.capitalize()} layers beside {'Zederax and ' if args.workload == 'nakurax' else ''}GPT-2 layers of equal width, heads and inner width"),
                       "unit": "tok/s", "n_gpus": 1, "steps": steps, "warmup": warmup, "dtype": "bf16" if args.dtype == "bfloat16" else "fp32",
                       "data": "synthetic (random weights, uniform-random token ids)", "results": results}), flush=True)
     return 0

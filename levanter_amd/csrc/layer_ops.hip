@@ -207,6 +207,95 @@ extern "C" int lev_norm_write_latent(void* c, long c_stride, int R, int norm_dim
   return lev_check_launch("norm_write_latent");
 }
 
+// The same for a latent with a rotated key part behind it, and the rotation of the queries, in one launch (steps of single
+// tokens). A token's row `kv` holds [c (R) | k_rot (DR)]: c becomes its RMS norm with the weight `w` (mean of squares over
+// norm_dim), in place; k_rot has dimension i < n_pairs paired with dimension i + n_pairs and each pair turned by
+// positions[t] * freqs[i], in place; the key pages (one key head of R + DR) take [c | k_rot], the value pages (one head of
+// R) take c. Every head of `q` (HQ heads of q_head elements) has the vector that starts q_off elements into it turned the
+// same way. The arithmetic is that of head_prepare, rotary_half and kv_write, one after the other.
+template <typename T>
+__global__ void __launch_bounds__(256)
+latent_rope_write_kernel(T* __restrict__ kv, long kv_stride, int R, int DR, int norm_dim, float eps, const float* __restrict__ w,
+                         T* __restrict__ q, long q_stride, int HQ, int q_head, int q_off, int n_pairs, const float* __restrict__ freqs,
+                         const int* __restrict__ positions, T* __restrict__ k_pages, T* __restrict__ v_pages, const int* __restrict__ dest,
+                         int PS) {
+  __shared__ float red[4];
+  const int t = blockIdx.x;
+  T* row = kv + (size_t)t * kv_stride;
+  const float p = (float)positions[t];
+  float ss = 0.f;
+  for (int d = threadIdx.x; d < R; d += 256) {
+    const float x = to_float<T>(row[d]);
+    ss = fmaf(x, x, ss);
+  }
+  ss = block_sum<256>(ss, red);
+  const float r = 1.0f / sqrtf(ss / (float)norm_dim + eps);
+  const int dst = dest[t];
+  const int KD = R + DR;
+  T* kd = k_pages + (size_t)max(dst, 0) / PS * (size_t)KD * PS;
+  T* vd = v_pages + (size_t)max(dst, 0) / PS * (size_t)R * PS;
+  const int off = max(dst, 0) % PS;
+  for (int d = threadIdx.x; d < R; d += 256) {
+    const T val = from_float<T>(to_float<T>(row[d]) * r * w[d]);
+    row[d] = val;
+    if (dst >= 0) {
+      kd[((size_t)(d >> 3) * PS + off) * 8 + (d & 7)] = val;
+      vd[(size_t)d * PS + off] = val;
+    }
+  }
+  // the rotated key part: pairs first, then what lies behind them unchanged
+  for (int i = threadIdx.x; i < DR; i += 256) {
+    if (i < n_pairs) {
+      float sn, cs;
+      sincosf(p * freqs[i], &sn, &cs);
+      const float a = to_float<T>(row[R + i]), b = to_float<T>(row[R + i + n_pairs]);
+      const T lo = from_float<T>(a * cs - b * sn), hi = from_float<T>(b * cs + a * sn);
+      row[R + i] = lo;
+      row[R + i + n_pairs] = hi;
+      if (dst >= 0) {
+        const int d0 = R + i, d1 = R + i + n_pairs;
+        kd[((size_t)(d0 >> 3) * PS + off) * 8 + (d0 & 7)] = lo;
+        kd[((size_t)(d1 >> 3) * PS + off) * 8 + (d1 & 7)] = hi;
+      }
+    } else if (i >= 2 * n_pairs && dst >= 0) {
+      const int d0 = R + i;
+      kd[((size_t)(d0 >> 3) * PS + off) * 8 + (d0 & 7)] = row[d0];
+    }
+  }
+  if (q != nullptr) {
+    const int items = HQ * n_pairs;
+    for (int it = threadIdx.x; it < items; it += 256) {
+      const int head = it / n_pairs, i = it - head * n_pairs;
+      T* v = q + (size_t)t * q_stride + (size_t)head * q_head + q_off;
+      float sn, cs;
+      sincosf(p * freqs[i], &sn, &cs);
+      const float a = to_float<T>(v[i]), b = to_float<T>(v[i + n_pairs]);
+      v[i] = from_float<T>(a * cs - b * sn);
+      v[i + n_pairs] = from_float<T>(b * cs + a * sn);
+    }
+  }
+}
+
+extern "C" int lev_latent_rope_write(void* kv, long kv_stride, int R, int DR, int norm_dim, float eps, const float* w, void* q, long q_stride,
+                                     int HQ, int q_head, int q_off, int n_pairs, const float* freqs, const int* positions, void* k_pages,
+                                     void* v_pages, const int* dest, int PS, int T, int dtype, hipStream_t stream) {
+  LEV_REQUIRE(T >= 0 && R > 0 && R % 8 == 0 && DR >= 0 && DR % 8 == 0 && norm_dim > 0 && norm_dim <= R && kv_stride >= R + DR,
+              "latent_rope_write: bad sizes T=%d R=%d of %d, rotated part %d", T, R, norm_dim, DR);
+  LEV_REQUIRE(n_pairs >= 0 && 2 * n_pairs <= DR && (n_pairs == 0 || (freqs && positions)), "latent_rope_write: %d pairs do not fit a rotated part of %d", n_pairs, DR);
+  LEV_REQUIRE(q == nullptr || (HQ > 0 && q_off >= 0 && q_off + 2 * n_pairs <= q_head && q_stride >= (long)HQ * q_head), "latent_rope_write: the queries' rotated part does not fit their heads");
+  LEV_REQUIRE(kv && w && k_pages && v_pages && dest && positions, "latent_rope_write: a tensor is missing");
+  LEV_REQUIRE(PS > 0 && PS % 16 == 0, "latent_rope_write: page_size=%d must be a multiple of 16", PS);
+  LEV_REQUIRE(dtype == LEV_F32 || dtype == LEV_BF16, "latent_rope_write: unknown dtype %d", dtype);
+  if (T == 0) return 0;
+  if (dtype == LEV_F32)
+    latent_rope_write_kernel<float><<<T, 256, 0, stream>>>((float*)kv, kv_stride, R, DR, norm_dim, eps, w, (float*)q, q_stride, HQ, q_head, q_off, n_pairs,
+                                                          freqs, positions, (float*)k_pages, (float*)v_pages, dest, PS);
+  else
+    latent_rope_write_kernel<bf16_t><<<T, 256, 0, stream>>>((bf16_t*)kv, kv_stride, R, DR, norm_dim, eps, w, (bf16_t*)q, q_stride, HQ, q_head, q_off,
+                                                           n_pairs, freqs, positions, (bf16_t*)k_pages, (bf16_t*)v_pages, dest, PS);
+  return lev_check_launch("latent_rope_write");
+}
+
 // ------------------------------------------------------------------------------------------
 // out = c0 z / rms(z) + c1 z^2 / rms(z^2) + c2 z^3 / rms(z^3) + c3 over a row of F values, rms(u) = sqrt(mean(u^2) + eps).
 // One block per row; the row is read twice (statistics, then the output), the second time from the cache. `out` may be `z`.

@@ -276,6 +276,7 @@ register_unit("core", ["errors.hip", "elementwise.hip", "layer_ops.hip", "gemm_s
     "lev_embed": [_P] * 5 + [_I, _I, _I, _F, _P],
     "lev_streams_step": [_P, _I, _I, _I, _P, _P, _P, _P, _P, _P, _F, _P, _P, _P, _I, _I, _P, _I, _P, _P],
     "lev_rotary_pairs": [_P, _L, _I, _P, _L, _I, _I, _I, _P, _P, _I, _I, _P],
+    "lev_latent_rope_write": [_P, _L, _I, _I, _I, _F, _P, _P, _L, _I, _I, _I, _I, _P, _P, _P, _P, _P, _I, _I, _I, _P],
     "lev_rotary_half": [_P, _L, _I, _I, _I, _I, _P, _P, _I, _I, _P],
     "lev_group_norm_step": [_P, _P, _P, _L, _I, _P, _F, _P, _P, _I, _P, _I, _I, _I, _F, _P],
     "lev_delta_rule": [_P] * 5 + [_L, _P, _L, _P, _P, _P, _P, _L, _I, _I, _I, _F, _F, _F, _I, _P],
@@ -327,5 +328,5 @@ for _hd in MFMA_ATTENTION_HEAD_DIMS:
         "lev_attention_mfma": [_P, _L, _P, _L, _P, _P, _P, _P, _P, _I, _P, _I, _P, _I, _P, _P, _L, _P, _P] + [_I] * 5 + [_F, _I, _F, _P, _I, _P],
     })
 # key / value head sizes of the attention with separate sizes that are built ahead; any other pair is built at its first use
-for _hd, _vd in ((32, 16), (16, 32), (48, 32), (64, 64), (128, 64), (128, 128), (256, 256), (32, 32), (16, 16)):
+for _hd, _vd in ((32, 16), (16, 32), (48, 32), (64, 64), (128, 64), (128, 128), (256, 256), (32, 32), (16, 16), (64, 48), (64, 32), (80, 64), (160, 128), (256, 224)):
     attention_values_unit(_hd, _vd)

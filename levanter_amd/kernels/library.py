@@ -506,6 +506,30 @@ class HipKernels:
         self._check(self.lib.lev_norm_write_latent(_ptr(c), _rows(c, "norm_write_latent: c"), R, int(norm_dim), float(eps), _ptr(weight), _ptr(k_pages),
                                                    _ptr(v_pages), _ptr(dest), page_size, T, _DT[c.dtype], self._s()))
 
+    def latent_rope_write(self, kv, latent_dim: int, weight, eps: float, norm_dim: int, q, n_heads: int, q_head: int, q_offset: int, freqs, positions,
+                          k_pages, v_pages, dest, page_size: int) -> None:
+        """For steps of single tokens, in one kernel: ``kv`` ``[T, latent_dim + rotated part]`` has its latent normed (``head_prepare``
+        with ``weight``, the mean of squares over ``norm_dim``) and its rotated part turned (``rotary_half`` from column
+        ``latent_dim``), in place; the whole row goes into the key pages and the latent into the value pages at ``dest``
+        (``kv_write``); the vectors at ``q_offset`` of the ``n_heads`` heads of ``q_head`` elements of ``q`` are turned too (``q`` None:
+        no queries). ``freqs`` float32 (may be empty: nothing turns)."""
+        _dev(kv, weight, q, freqs, positions, k_pages, v_pages, dest)
+        T, KD = kv.shape
+        R, DR = int(latent_dim), KD - int(latent_dim)
+        dt = kv.dtype
+        _req(dt in _DT and dt == k_pages.dtype == v_pages.dtype and (q is None or q.dtype == dt), "latent_rope_write: dtypes differ")
+        _req(weight.dtype == torch.float32 and weight.numel() == R and weight.is_contiguous(), "latent_rope_write: the weight must be float32 [latent_dim]")
+        _req(freqs is None or (freqs.dtype == torch.float32 and freqs.is_contiguous()), "latent_rope_write: float32 frequencies")
+        n_pairs = 0 if freqs is None else freqs.numel()
+        _req(positions.dtype == torch.int32 and positions.numel() == T and dest.dtype == torch.int32 and dest.numel() == T, "latent_rope_write: one int32 position and destination per token")
+        _req(k_pages.is_contiguous() and v_pages.is_contiguous() and k_pages.numel() * R == v_pages.numel() * KD and k_pages.numel() % (KD * page_size) == 0,
+             "latent_rope_write: page tensors must be contiguous and fit the sizes")
+        _req(q is None or (q.dim() == 2 and q.shape[0] == T and q.shape[1] >= n_heads * q_head), "latent_rope_write: q must be [T, heads*q_head]")
+        self._check(self.lib.lev_latent_rope_write(_ptr(kv), _rows(kv, "latent_rope_write: kv"), R, DR, int(norm_dim), float(eps), _ptr(weight), _ptr(q),
+                                                   _rows(q, "latent_rope_write: q") if q is not None else 0, int(n_heads), int(q_head), int(q_offset), n_pairs,
+                                                   _ptr(freqs) if n_pairs else None, _ptr(positions), _ptr(k_pages), _ptr(v_pages), _ptr(dest), page_size, T,
+                                                   _DT[dt], self._s()))
+
     def recurrent_tokens(self, x, y, taps, conv_bias, gate_weight, gate_bias, decay, state, token_slots, out, out_scale: float = 1.0) -> None:
         """``causal_conv``, the block-diagonal product of the gates and ``gated_recurrence`` for a step in which every token is
         a run of its own, in one kernel (the same bits as the three). ``gate_weight`` ``[B, 2*C/B, C/B]``: both gates of a block
@@ -807,6 +831,8 @@ class HipKernels:
         _req(freqs.dtype == torch.float32 and freqs.is_contiguous() and offset >= 0 and offset + 2 * freqs.numel() <= head_stride,
              "rotary: float32 frequencies, and the rotated vector must fit the head")
         _req(positions.dtype == torch.int32 and positions.numel() == T, "rotary: one int32 position per token")
+        if freqs.numel() == 0:
+            return
         self._check(self.lib.lev_rotary_half(_ptr(x), _rows(x, "rotary: x"), int(n_heads), int(head_stride), int(offset), freqs.numel(), _ptr(freqs),
                                              _ptr(positions), T, _DT[x.dtype], self._s()))
 

@@ -85,7 +85,7 @@ class GeneralDeltaRule(Mixer):
         self.attend(self.proj(h, ctx), ctx, unit, writes_cache, a, h)
         self.out(a, ctx, out=y, may_leave=True)
 
-    def attend(self, p: torch.Tensor, ctx: StepContext, unit: CacheUnitView, writes_cache: bool, a: torch.Tensor, h: torch.Tensor) -> None:
+    def attend(self, p: torch.Tensor, ctx: StepContext, unit: CacheUnitView, writes_cache: bool, a: torch.Tensor, h: torch.Tensor = None) -> None:
         """Everything between the two products: ``p`` ``[T, r | k | v | removal | gate (| columns of others)]`` is what ``proj`` gives,
         ``h`` the mixer's input (for the decay's own products), ``a`` ``[T, H*d]`` takes what ``out`` reads. The request's state is
         read and advanced."""

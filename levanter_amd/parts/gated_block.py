@@ -72,6 +72,22 @@ class GatedPostNorm(Part):
         """``gate.weight h + gate.bias`` (the sigmoid is taken where the gate is applied)."""
         return None if self.gate is None else self.gate(h, ctx)
 
+    def fuse_behind(self, first: Linear, env: BuildEnv) -> Optional[Linear]:
+        """One product for ``first`` and the gate, which read the same input: ``[first's rows | zeros up to a multiple of 8 | gate]``.
+        The connection drops its own matrix; whoever runs the product hands the gate's columns (from ``gate_offset``) to ``write``.
+        None if there is no gate or the two do not fit together."""
+        if self.gate is None or first.weight.dtype != self.gate.weight.dtype or first.n_in != self.dim:
+            return None
+        dev = first.weight.device
+        fill = (-first.n_out) % 8
+        self.gate_offset = first.n_out + fill
+        zeros = torch.zeros(fill, self.dim, dtype=first.weight.dtype, device=dev)
+        b1 = first.bias if first.bias is not None else torch.zeros(first.n_out, device=dev)
+        b2 = self.gate.bias if self.gate.bias is not None else torch.zeros(self.dim, device=dev)
+        fused = Linear(torch.cat([first.weight, zeros, self.gate.weight], 0), torch.cat([b1, torch.zeros(fill, device=dev), b2]), "out_in", env)
+        self.gate = None
+        return fused
+
     def write(self, y: torch.Tensor, gate: Optional[torch.Tensor], x: torch.Tensor, ctx: StepContext) -> None:
         pending = ctx.kernels.group_norm_step(x, groups=self.groups, eps=self.eps, y=y, gate=gate, post_weight=self.weight, mult=self.mult, defer=True)
         if ctx.may_defer:
@@ -98,23 +114,58 @@ class GatedSandwichBlock(Block):
         self.norm2, self.connect2 = parts.get("norm2"), parts.get("connect2")
         if self.feed_forward is not None and (self.norm2 is None or self.connect2 is None):
             raise ValueError("block 'gated_sandwich': a feed-forward needs norm2 and connect2")
+        # a sublayer's gate reads the sublayer's own input: where the sublayer offers its first product (a mixer's ``proj`` with
+        # ``attend`` and ``out``, a feed-forward's ``router`` with ``run_routed``), the gate's rows join it and the parts drop theirs
+        self.fused_mixer = self.fused_ff = None
+        m, f = self.mixer, self.feed_forward
+        if all(hasattr(m, a) for a in ("proj", "attend", "out")) and hasattr(self.connect1, "fuse_behind"):
+            self.mixer_cols = m.proj.n_out
+            self.fused_mixer = self.connect1.fuse_behind(m.proj, m.env)
+            if self.fused_mixer is not None:
+                m.proj = None
+        if f is not None and all(hasattr(f, a) for a in ("router", "run_routed")) and hasattr(self.connect2, "fuse_behind"):
+            self.router_cols = f.router.n_out
+            self.fused_ff = self.connect2.fuse_behind(f.router, f.env)
+            if self.fused_ff is not None:
+                f.router = None
 
     def _sublayer(self, norm, connect, run, x: torch.Tensor, ctx: StepContext) -> None:
+        """``run(h, y)`` computes the sublayer's result into ``y`` and gives the gate's sums if its first product has made them."""
         may_defer = ctx.may_defer
         if not norm.folds_pending:
             ctx.settle()
         h = norm(x, ctx)
         y = torch.empty_like(x)
         ctx.may_defer = False  # a sublayer's result is complete before it is gated and normed
-        run(h, y)
+        gate = run(h, y)
         product = ctx.take_product_pending(y)
         if product is not None:
             ctx.kernels.finish(product)
-        gate = connect.gate_of(h, ctx)
+        if gate is None:
+            gate = connect.gate_of(h, ctx)
         ctx.may_defer = may_defer
         connect.write(y, gate, x, ctx)
 
+    def _run_mixer(self, h, y, ctx, unit, writes_cache):
+        if self.fused_mixer is None:
+            self.mixer.compute(h, y, ctx, unit, writes_cache)
+            return None
+        m = self.mixer
+        pz = self.fused_mixer(h, ctx)  # [T, the mixer's projections | the gate]
+        a = ctx.empty(h.shape[0], m.out.n_in)
+        m.attend(pz[:, :self.mixer_cols], ctx, unit, writes_cache, a, h=h)
+        m.out(a, ctx, out=y)
+        return pz[:, self.connect1.gate_offset:self.connect1.gate_offset + self.connect1.dim]
+
+    def _run_feed_forward(self, h, y, ctx):
+        if self.fused_ff is None:
+            self.feed_forward.compute(h, y, ctx)
+            return None
+        pz = self.fused_ff(h, ctx, out_dtype=torch.float32)  # the router's logits are 32-bit sums, so the gate's are too
+        self.feed_forward.run_routed(h, pz[:, :self.router_cols], y, ctx)
+        return pz[:, self.connect2.gate_offset:self.connect2.gate_offset + self.connect2.dim]
+
     def forward(self, x: torch.Tensor, ctx: StepContext, unit: CacheUnitView, writes_cache: bool) -> None:
-        self._sublayer(self.norm1, self.connect1, lambda h, y: self.mixer.compute(h, y, ctx, unit, writes_cache), x, ctx)
+        self._sublayer(self.norm1, self.connect1, lambda h, y: self._run_mixer(h, y, ctx, unit, writes_cache), x, ctx)
         if self.feed_forward is not None:
-            self._sublayer(self.norm2, self.connect2, lambda h, y: self.feed_forward.compute(h, y, ctx), x, ctx)
+            self._sublayer(self.norm2, self.connect2, lambda h, y: self._run_feed_forward(h, y, ctx), x, ctx)

@@ -145,9 +145,9 @@ class LatentAttention(Mixer):
         self.attend(self.proj(h, ctx), ctx, unit, writes_cache, a)
         self.out(a, ctx, out=y, may_leave=True)
 
-    def attend(self, p: torch.Tensor, ctx: StepContext, unit: CacheUnitView, writes_cache: bool, a: torch.Tensor) -> None:
+    def attend(self, p: torch.Tensor, ctx: StepContext, unit: CacheUnitView, writes_cache: bool, a: torch.Tensor, h=None) -> None:
         """Everything between the two products: ``p`` ``[T, q | latent (| columns of others)]`` is what ``proj`` gives, ``a``
-        ``[T, heads * value_dim]`` (rows may be strided) takes the heads that ``out`` reads."""
+        ``[T, heads * value_dim]`` (rows may be strided) takes the heads that ``out`` reads. (``h``, the mixer's input, is not needed.)"""
         K = ctx.kernels
         T, H, Rp, KD = p.shape[0], self.n_heads, self.latent, self.key_dim
         g = unit.group
@@ -159,17 +159,21 @@ class LatentAttention(Mixer):
             q = self.up_q(p[:, :self.q_latent], ctx)
         else:
             q = p[:, :self.q_cols]
-        if self.freqs is not None:
+        singles = ctx.attention.n_prefill_tiles == 0  # a step of single tokens: rotation, norm and cache write in one kernel
+        if self.freqs is not None and not (singles and writes_cache and self.rope):
             K.rotary_half(q, H, self.q_head, self.head_dim, self.freqs, positions)
         if writes_cache:
             kv = p[:, self.c_off:self.c_off + KD]  # [latent | rotated key part]
             c = kv[:, :Rp]
-            if self.freqs is not None:
-                K.rotary_half(kv, 1, KD, Rp, self.freqs, positions)
-            # the latent's RMS norm, in place; then into the pages, as key and as value
-            if self.rope == 0 and ctx.attention.n_prefill_tiles == 0:  # a step of single tokens: both in one kernel
+            if singles and self.rope:
+                K.latent_rope_write(kv, Rp, self.norm_weight, self.eps, self.true_latent, q, H, self.q_head, self.head_dim, self.freqs, positions,
+                                    unit.k_pages, unit.v_pages, g.dest, g.page_size)
+            elif singles:
                 K.norm_write_latent(c, self.norm_weight, self.eps, self.true_latent, unit.k_pages, unit.v_pages, g.dest, g.page_size)
             else:
+                if self.freqs is not None:
+                    K.rotary_half(kv, 1, KD, Rp, self.freqs, positions)
+                # the latent's RMS norm (32-bit statistics, the weight applied), in place; then into the pages, as key and as value
                 K.head_prepare(c, 1, Rp, self.eps, norm_dim=self.true_latent, norm_weight=self.norm_weight)
                 K.kv_write(kv, c, unit.k_pages, unit.v_pages, g.dest, 1, KD, g.page_size, value_dim=Rp)  # 16 tokens at a time, transposed through LDS
         qa = ctx.empty(T, H * KD)

@@ -72,11 +72,17 @@ class RoutedExperts(FeedForward):
     def compute(self, h: torch.Tensor, y: torch.Tensor, ctx: StepContext) -> None:
         self._run(h, y, ctx, False)
 
-    def _run(self, h: torch.Tensor, y: torch.Tensor, ctx: StepContext, accumulate: bool) -> None:
+    def run_routed(self, h: torch.Tensor, z: torch.Tensor, y: torch.Tensor, ctx: StepContext) -> None:
+        """The feed-forward's result into ``y`` from router logits ``z`` (float32 ``[T, E]``, rows may be strided) that a block has
+        computed as part of a larger product over ``h``."""
+        self._run(h, y, ctx, False, z)
+
+    def _run(self, h: torch.Tensor, y: torch.Tensor, ctx: StepContext, accumulate: bool, z=None) -> None:
         K = ctx.kernels
         T, E, top = h.shape[0], self.n_experts, self.top
         dev = h.device
-        z = self.router(h, ctx, out_dtype=torch.float32)
+        if z is None:
+            z = self.router(h, ctx, out_dtype=torch.float32)
         if accumulate:
             ctx.settle()  # the sum below reads the residual stream itself
         chosen = torch.empty((T, top), dtype=torch.int32, device=dev)

@@ -409,6 +409,16 @@ class EmulatedKernels:
         self.head_prepare(c, 1, c.shape[1], eps, norm_dim=norm_dim, norm_weight=weight)
         self.kv_write(c, c, k_pages, v_pages, dest, 1, c.shape[1], page_size)
 
+    def latent_rope_write(self, kv, latent_dim, weight, eps, norm_dim, q, n_heads, q_head, q_offset, freqs, positions, k_pages, v_pages, dest,
+                          page_size) -> None:
+        KD = kv.shape[1]
+        self.head_prepare(kv, 1, latent_dim, eps, norm_dim=norm_dim, norm_weight=weight)
+        if freqs is not None and freqs.numel():
+            self.rotary_half(kv, 1, KD, latent_dim, freqs, positions)
+            if q is not None:
+                self.rotary_half(q, n_heads, q_head, q_offset, freqs, positions)
+        self.kv_write(kv, kv[:, :latent_dim], k_pages, v_pages, dest, 1, KD, page_size, value_dim=latent_dim)
+
     def recurrent_tokens(self, x, y, taps, conv_bias, gate_weight, gate_bias, decay, state, token_slots, out, out_scale=1.0) -> None:
         u = torch.empty_like(x)
         self.causal_conv(x, taps, conv_bias, state, token_slots, u)

@@ -155,10 +155,32 @@ def expert(h: torch.Tensor, W: Dict[str, torch.Tensor], p: str) -> torch.Tensor:
     return ((g * torch.sigmoid(g)) * (h @ W[f"{p}.up"].T)) @ W[f"{p}.down"].T
 
 
-def moe(h: torch.Tensor, W: Dict[str, torch.Tensor], p: str, mlp: dict) -> torch.Tensor:
+def route_margin(z: torch.Tensor, correction: torch.Tensor, top: int, n_groups: int, keep: int) -> torch.Tensor:
+    """Per token, how far the router's choice is from another one: the gap in choice score between the last expert taken and
+    the best one left out, and between the last group kept and the best one dropped; infinite where there is no choice."""
+    T, E = z.shape
+    choice = torch.sigmoid(z) + correction
+    per = E // n_groups
+    out = torch.full((T,), math.inf, dtype=F64)
+    group_score = choice.view(T, n_groups, per).topk(min(2, per), -1).values.sum(-1)
+    allowed = torch.ones(T, n_groups, dtype=torch.bool)
+    if keep < n_groups:
+        best = group_score.topk(keep + 1, -1)
+        out = torch.minimum(out, best.values[:, keep - 1] - best.values[:, keep])
+        allowed = torch.zeros(T, n_groups, dtype=torch.bool).scatter_(1, best.indices[:, :keep], True)
+    if top < keep * per:
+        masked = choice.masked_fill(~allowed[:, :, None].expand(T, n_groups, per).reshape(T, E), -math.inf)
+        best = masked.topk(top + 1, -1).values
+        out = torch.minimum(out, best[:, top - 1] - best[:, top])
+    return out
+
+
+def moe(h: torch.Tensor, W: Dict[str, torch.Tensor], p: str, mlp: dict, margins: Optional[list] = None) -> torch.Tensor:
     r = mlp["router"]
     groups = r.get("groups") or {"count": 1, "keep": 1}
     chosen, weights = route(h @ W[f"{p}.router"].T, W[f"{p}.correction"], r["top"], groups["count"], groups["keep"])
+    if margins is not None:
+        margins.append(route_margin(h @ W[f"{p}.router"].T, W[f"{p}.correction"], r["top"], groups["count"], groups["keep"]))
     out = torch.zeros_like(h)
     for t in range(h.shape[0]):
         for e, wt in zip(chosen[t].tolist(), weights[t]):
@@ -167,8 +189,9 @@ def moe(h: torch.Tensor, W: Dict[str, torch.Tensor], p: str, mlp: dict) -> torch
 
 
 # ---- the model ----------------------------------------------------------------------------------------------------
-def forward(cfg: dict, W: Dict[str, torch.Tensor], tokens: List[int], return_layers: bool = False):
-    """Logits ``[T, vocab]`` of one whole sequence (and the residual stream after every layer)."""
+def forward(cfg: dict, W: Dict[str, torch.Tensor], tokens: List[int], return_layers: bool = False, margins: Optional[list] = None):
+    """Logits ``[T, vocab]`` of one whole sequence (and the residual stream after every layer). ``margins``: a list that takes
+    every routed layer's ``route_margin``."""
     eps, groups, mult = float(cfg["norm"]["eps"]), int(cfg["norm"]["groups"]), float(cfg["residual_mult"])
 
     def norm(x, name):
@@ -193,7 +216,7 @@ def forward(cfg: dict, W: Dict[str, torch.Tensor], tokens: List[int], return_lay
         x = x + mult * norm(y, f"{p}.norm1b")
         if layer.get("mlp") is not None:
             h = norm(x, f"{p}.norm2")
-            y = moe(h, W, f"{p}.mlp", layer["mlp"])
+            y = moe(h, W, f"{p}.mlp", layer["mlp"], margins)
             y = y * torch.sigmoid(h @ W[f"{p}.rg2"].T + W[f"{p}.rg2.b"])
             x = x + mult * norm(y, f"{p}.norm2b")
         after.append(x)
@@ -203,6 +226,18 @@ def forward(cfg: dict, W: Dict[str, torch.Tensor], tokens: List[int], return_lay
 
 def plain_logits(W: Dict[str, torch.Tensor], cfg: dict, tokens) -> torch.Tensor:
     return forward(cfg, W, [int(t) for t in tokens])
+
+
+def first_close_call(W: Dict[str, torch.Tensor], cfg: dict, tokens, delta: float) -> int:
+    """The first position at which some layer's router decides by less than ``delta`` (the sequence's length if none does). In
+    16-bit arithmetic such a choice may fall the other way: that token's result is then another model's, and so is, through
+    caches and states, every later token's. Nothing that a test asserts may rest on such a position."""
+    margins: list = []
+    forward(cfg, W, [int(t) for t in tokens], margins=margins)
+    if not margins:
+        return len(tokens)
+    close = (torch.stack(margins).min(0).values < delta).nonzero().flatten()
+    return int(close[0]) if close.numel() else len(tokens)
 
 
 def plain_greedy(W: Dict[str, torch.Tensor], cfg: dict, prompt: List[int], n_new: int) -> List[int]:
@@ -241,10 +276,12 @@ def make_config(vocab=97, width=64, layers=None, eps=1e-5, groups=2, mult=0.7) -
     return {"architecture": "Tativik", "vocab": vocab, "width": width, "norm": {"eps": eps, "groups": groups}, "residual_mult": mult, "layers": layers}
 
 
-def random_weights(cfg: dict, seed: int, dtype=F64) -> Dict[str, torch.Tensor]:
+def random_weights(cfg: dict, seed: int, dtype=F64, clear_routing: bool = False) -> Dict[str, torch.Tensor]:
     """Weights drawn so that every mechanism matters: scores of order one, sinks that take a visible share of the weight,
     gates that are not saturated, decays and removal rates over their whole range, router scores whose order the correction
-    changes. Values are bfloat16 numbers (a file stores them exactly)."""
+    changes. Values are bfloat16 numbers (a file stores them exactly). ``clear_routing``: routers that decide by a wide margin
+    (scores near one half that move a little with the input, corrections drawn until every border of the choice has a wide gap), for runs in 16-bit
+    arithmetic, where a choice by less than the inputs' rounding could fall either way."""
     g = torch.Generator().manual_seed(seed)
     D, V = cfg["width"], cfg["vocab"]
 
@@ -289,8 +326,15 @@ def random_weights(cfg: dict, seed: int, dtype=F64) -> Dict[str, torch.Tensor]:
                 W[p + n] = 1 + rn(D, std=0.2)
             W[p + "rg2"] = rn(D, D, std=1 / math.sqrt(D))
             W[p + "rg2.b"] = rn(D, std=0.5)
-            W[p + "mlp.router"] = rn(E, D, std=1.5 / math.sqrt(D))
+            W[p + "mlp.router"] = rn(E, D, std=(0.05 if clear_routing else 1.5) / math.sqrt(D))
             W[p + "mlp.correction"] = rn(E, std=0.3)
+            while clear_routing:  # corrections that leave a wide gap at every border of the choice, between groups too
+                corr = (torch.rand(E, generator=g) * 0.3 * E - 0.5).to(torch.bfloat16).to(dtype)
+                r = mlp["router"]
+                gr = r.get("groups") or {"count": 1, "keep": 1}
+                if float(route_margin(torch.zeros(1, E, dtype=dtype), corr, r["top"], gr["count"], gr["keep"])[0]) >= 0.15:
+                    W[p + "mlp.correction"] = corr
+                    break
             for e in range(E):
                 W[p + f"mlp.e{e}.gate"] = rn(F, D, std=1 / math.sqrt(D))
                 W[p + f"mlp.e{e}.up"] = rn(F, D, std=1 / math.sqrt(D))

@@ -45,30 +45,29 @@ group_norm_step_kernel(float* __restrict__ x, const float* __restrict__ y, const
   const int r = blockIdx.x, row = rows ? rows[r] : r;
   const int group_size = D / G;
   const float inv_n = 1.0f / (float)group_size;
-  float xv[PER];
+  float xv[PER], z[PER], pw[PER], wv[PER];
   int gid[PER];  // the group of each of this thread's elements; -1 beyond the row
+  // every load of the row is asked for before anything is computed: the kernel is a chain of a few memory latencies otherwise
 #pragma unroll
   for (int i = 0; i < PER; ++i) {
-    const int e = tid + GN_NT * i;
-    xv[i] = e < D ? x[(size_t)row * D + e] : 0.f;
+    const int e = tid + GN_NT * i, ec = min(e, D - 1);
+    xv[i] = x[(size_t)row * D + ec];
+    z[i] = y != nullptr ? y[(size_t)row * D + ec] : 0.f;
+    pw[i] = y != nullptr ? post_w[ec] : 0.f;
+    wv[i] = h_out != nullptr ? w[ec] : 0.f;
+    const float gt = gate != nullptr ? to_float<TG>(gate[(size_t)row * gate_stride + ec]) : 0.f;
+    if (gate != nullptr) z[i] = z[i] / (1.0f + expf(-gt));
+    if (e >= D) xv[i] = 0.f, z[i] = 0.f;
     gid[i] = e < D ? e / group_size : -1;
   }
   if (y != nullptr) {
-    float z[PER];
-#pragma unroll
-    for (int i = 0; i < PER; ++i) {
-      const int e = tid + GN_NT * i;
-      float v = e < D ? y[(size_t)row * D + e] : 0.f;
-      if (gate != nullptr && e < D) v = v / (1.0f + expf(-to_float<TG>(gate[(size_t)row * gate_stride + e])));
-      z[i] = v;
-    }
     group_square_sums<PER>(z, gid, G, part, total);
 #pragma unroll
     for (int i = 0; i < PER; ++i) {
       const int e = tid + GN_NT * i;
       if (e < D) {
         const float inv = 1.0f / sqrtf(total[gid[i]] * inv_n + eps);
-        xv[i] = xv[i] + mult * (z[i] * inv * post_w[e]);
+        xv[i] = xv[i] + mult * (z[i] * inv * pw[i]);
         if (rows == nullptr) x[(size_t)row * D + e] = xv[i];
       }
     }
@@ -81,7 +80,7 @@ group_norm_step_kernel(float* __restrict__ x, const float* __restrict__ y, const
       const int e = tid + GN_NT * i;
       if (e < D) {
         const float inv = 1.0f / sqrtf(total[gid[i]] * inv_n + eps);
-        h_out[(size_t)r * D + e] = from_float<TO>(xv[i] * inv * w[e]);
+        h_out[(size_t)r * D + e] = from_float<TO>(xv[i] * inv * wv[i]);
       }
     }
   }

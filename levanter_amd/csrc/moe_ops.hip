@@ -6,7 +6,9 @@
 //             experts of the `keep` best groups can be chosen (the others count as -inf); the `top` largest c win (ties: the
 //             lower index); the weights are the winners' s (times 1 / their sum if `renormalize`), in the order of falling c.
 //   sort      the T * top (token, choice) pairs by expert: sorted[pos] = pair, pos_of[pair] = pos, and a list of row tiles
-//             (expert, first position, rows <= MOE_TM) that covers every expert's stretch; n_tiles on the device.
+//             (expert, first position, rows <= tile_rows) that covers every expert's stretch; n_tiles on the device.
+//             tile_rows is 16, or 64 for steps with many rows an expert (a wave then runs four row tiles on every weight
+//             fragment it loads).
 //   linear    for every tile: out[pos][o] = sum_k w[expert][o][k] a[row(pos)][k], row(pos) = the pair's token (gather) or pos
 //             itself; with glu the expert's matrix is [gate ; up] (2F rows) and out[pos][f] = act(gate_f) * up_f.
 //             bfloat16 on the matrix cores (16x16x32, both operands straight from global memory, as the block-diagonal
@@ -14,7 +16,7 @@
 //   combine   y[t] = sum_c weight[t][c] * out[pos_of[t * top + c]], c in order, float32; with `accumulate` added to what y holds.
 #include "common.h"
 
-#define MOE_TM 16          // rows of a tile
+#define MOE_TM 16          // rows of a matrix-core row tile; a tile of the list has tile_rows = MOE_TM or 4 * MOE_TM rows
 #define MOE_MAX_E 1024     // experts
 #define MOE_MAX_TOP 32
 
@@ -104,8 +106,8 @@ extern "C" int lev_moe_route(const float* z, long z_stride, const float* correct
 // themselves is whatever the atomic counters give: a pair's results do not depend on its place in a tile.
 #define MOE_SORT_NT 1024
 __global__ void __launch_bounds__(MOE_SORT_NT)
-moe_sort_kernel(const int* __restrict__ chosen, int P, int E, int* __restrict__ sorted, int* __restrict__ pos_of, int* __restrict__ tiles,
-                int* __restrict__ meta) {
+moe_sort_kernel(const int* __restrict__ chosen, int P, int E, int tile_rows, int* __restrict__ sorted, int* __restrict__ pos_of,
+                int* __restrict__ tiles, int* __restrict__ meta) {
   __shared__ int count[MOE_MAX_E], start[MOE_MAX_E], tile_start[MOE_MAX_E + 1], cursor[MOE_MAX_E];
   const int tid = threadIdx.x;
   for (int e = tid; e < E; e += MOE_SORT_NT) count[e] = 0, cursor[e] = 0;
@@ -118,7 +120,7 @@ moe_sort_kernel(const int* __restrict__ chosen, int P, int E, int* __restrict__ 
       start[e] = at;
       tile_start[e] = tile;
       at += count[e];
-      tile += (count[e] + MOE_TM - 1) / MOE_TM;
+      tile += (count[e] + tile_rows - 1) / tile_rows;
     }
     tile_start[E] = tile;
     meta[0] = tile;
@@ -135,18 +137,19 @@ moe_sort_kernel(const int* __restrict__ chosen, int P, int E, int* __restrict__ 
     for (int i = 0; i < n; ++i) {
       int* tl = tiles + 3 * (size_t)(tile_start[e] + i);
       tl[0] = e;
-      tl[1] = start[e] + i * MOE_TM;
-      tl[2] = min(MOE_TM, count[e] - i * MOE_TM);
+      tl[1] = start[e] + i * tile_rows;
+      tl[2] = min(tile_rows, count[e] - i * tile_rows);
     }
   }
 }
 
-extern "C" int lev_moe_max_tiles(int P, int E) { return P / MOE_TM + E + 1; }
+extern "C" int lev_moe_max_tiles(int P, int E, int tile_rows) { return P / tile_rows + E + 1; }
 
-extern "C" int lev_moe_sort(const int* chosen, int P, int E, int* sorted, int* pos_of, int* tiles, int* meta, hipStream_t stream) {
+extern "C" int lev_moe_sort(const int* chosen, int P, int E, int tile_rows, int* sorted, int* pos_of, int* tiles, int* meta, hipStream_t stream) {
   LEV_REQUIRE(P >= 0 && E > 0 && E <= MOE_MAX_E, "experts: %d experts (at most %d)", E, MOE_MAX_E);
+  LEV_REQUIRE(tile_rows == MOE_TM || tile_rows == 4 * MOE_TM, "experts: tiles of %d rows (%d or %d)", tile_rows, MOE_TM, 4 * MOE_TM);
   LEV_REQUIRE(chosen && sorted && pos_of && tiles && meta, "experts: a tensor is missing");
-  moe_sort_kernel<<<1, MOE_SORT_NT, 0, stream>>>(chosen, P, E, sorted, pos_of, tiles, meta);
+  moe_sort_kernel<<<1, MOE_SORT_NT, 0, stream>>>(chosen, P, E, tile_rows, sorted, pos_of, tiles, meta);
   return lev_check_launch("moe_sort");
 }
 
@@ -162,19 +165,21 @@ moe_linear_plain_kernel(const T* __restrict__ a, long a_stride, const T* __restr
   const int tile = blockIdx.x;
   if (tile >= meta[0]) return;
   const int e = tiles[3 * tile], first = tiles[3 * tile + 1], rows = tiles[3 * tile + 2];
-  const int rr = threadIdx.x >> 4, o = blockIdx.y * 16 + (threadIdx.x & 15);
-  if (rr >= rows || o >= F) return;
-  const int pos = first + rr;
-  const T* ar = a + (size_t)(gather ? sorted[pos] / top : pos) * a_stride;
-  const T* wg = w + ((size_t)e * N + o) * K;
-  float acc = 0.f, acc_up = 0.f;
-  for (int kk = 0; kk < K; ++kk) acc = fmaf(to_float<T>(wg[kk]), to_float<T>(ar[kk]), acc);
-  if (glu) {
-    const T* wu = wg + (size_t)F * K;
-    for (int kk = 0; kk < K; ++kk) acc_up = fmaf(to_float<T>(wu[kk]), to_float<T>(ar[kk]), acc_up);
-    acc = moe_act(acc, acc_up, act);
+  const int o = blockIdx.y * 16 + (threadIdx.x & 15);
+  if (o >= F) return;
+  for (int rr = threadIdx.x >> 4; rr < rows; rr += 16) {  // a tile may have more rows than the workgroup has row threads
+    const int pos = first + rr;
+    const T* ar = a + (size_t)(gather ? sorted[pos] / top : pos) * a_stride;
+    const T* wg = w + ((size_t)e * N + o) * K;
+    float acc = 0.f, acc_up = 0.f;
+    for (int kk = 0; kk < K; ++kk) acc = fmaf(to_float<T>(wg[kk]), to_float<T>(ar[kk]), acc);
+    if (glu) {
+      const T* wu = wg + (size_t)F * K;
+      for (int kk = 0; kk < K; ++kk) acc_up = fmaf(to_float<T>(wu[kk]), to_float<T>(ar[kk]), acc_up);
+      acc = moe_act(acc, acc_up, act);
+    }
+    out[(size_t)pos * o_stride + o] = from_float<TO>(acc);
   }
-  out[(size_t)pos * o_stride + o] = from_float<TO>(acc);
 }
 
 typedef __attribute__((ext_vector_type(8))) __bf16 moe_bf16x8;
@@ -186,9 +191,10 @@ __device__ __forceinline__ moe_bf16x8 moe_as_bf16x8(moe_u32x4 v) {
   return c.b;
 }
 
-// bfloat16 on the matrix cores: a wave owns the tile's 16 rows and NT tiles of 16 outputs (with glu: of gate and of up);
-// the transposed product out^T = w a^T leaves each lane with four neighbouring outputs of one row.
-template <typename TO, int NT, bool GLU>
+// bfloat16 on the matrix cores: a wave owns the tile's rows (RT row tiles of 16) and NT tiles of 16 outputs (with glu: of gate
+// and of up); the transposed product out^T = w a^T leaves each lane with four neighbouring outputs of one row. Every weight
+// fragment a wave loads is used for all its row tiles.
+template <typename TO, int NT, bool GLU, int RT>
 __global__ void __launch_bounds__(256)
 moe_linear_mfma_kernel(const bf16_t* __restrict__ a, long a_stride, const bf16_t* __restrict__ w, TO* __restrict__ out, long o_stride,
                        const int* __restrict__ tiles, const int* __restrict__ meta, const int* __restrict__ sorted, int top, int gather,
@@ -199,20 +205,30 @@ moe_linear_mfma_kernel(const bf16_t* __restrict__ a, long a_stride, const bf16_t
   const int o0 = (blockIdx.y * 4 + wave) * 16 * NT;
   if (o0 >= F) return;  // the whole wave
   const int e = tiles[3 * tile], first = tiles[3 * tile + 1], rows = tiles[3 * tile + 2];
-  const int pos = first + min(col, rows - 1);  // rows beyond the tile: read again, never stored
-  const bf16_t* ar = a + (size_t)(gather ? sorted[pos] / top : pos) * a_stride;
+  const bf16_t* ar[RT];
+#pragma unroll
+  for (int rt = 0; rt < RT; ++rt) {
+    const int pos = first + min(16 * rt + col, rows - 1);  // rows beyond the tile: read again, never stored
+    ar[rt] = a + (size_t)(gather ? sorted[pos] / top : pos) * a_stride;
+  }
   const bf16_t* we = w + (size_t)e * N * K;
   const bf16_t* wr[NT];
 #pragma unroll
   for (int nt = 0; nt < NT; ++nt) wr[nt] = we + (size_t)min(o0 + 16 * nt + col, F - 1) * K;
-  moe_f32x4 acc[NT], acc_up[NT];
+  moe_f32x4 acc[RT][NT], acc_up[RT][NT];
 #pragma unroll
-  for (int nt = 0; nt < NT; ++nt) acc[nt] = acc_up[nt] = moe_f32x4{0.f, 0.f, 0.f, 0.f};
+  for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt) acc[rt][nt] = acc_up[rt][nt] = moe_f32x4{0.f, 0.f, 0.f, 0.f};
   for (int k0 = 0; k0 < K; k0 += 32) {
     const int kk = k0 + 8 * g, kc = min(kk, K - 8);  // loads stand under no condition; a chunk beyond the row counts as zeros
-    moe_u32x4 av = *reinterpret_cast<const moe_u32x4*>(ar + kc);
     const uint32_t keep = kk < K ? 0xffffffffu : 0u;
-    av = moe_u32x4{av[0] & keep, av[1] & keep, av[2] & keep, av[3] & keep};
+    moe_u32x4 av[RT];
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt) {
+      const moe_u32x4 x = *reinterpret_cast<const moe_u32x4*>(ar[rt] + kc);
+      av[rt] = moe_u32x4{x[0] & keep, x[1] & keep, x[2] & keep, x[3] & keep};
+    }
     moe_u32x4 wv[NT], wu[NT];
 #pragma unroll
     for (int nt = 0; nt < NT; ++nt) {
@@ -220,28 +236,35 @@ moe_linear_mfma_kernel(const bf16_t* __restrict__ a, long a_stride, const bf16_t
       if (GLU) wu[nt] = *reinterpret_cast<const moe_u32x4*>(wr[nt] + (size_t)F * K + kc);
     }
 #pragma unroll
-    for (int nt = 0; nt < NT; ++nt) {
-      acc[nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(moe_as_bf16x8(wv[nt]), moe_as_bf16x8(av), acc[nt], 0, 0, 0);
-      if (GLU) acc_up[nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(moe_as_bf16x8(wu[nt]), moe_as_bf16x8(av), acc_up[nt], 0, 0, 0);
-    }
+    for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+      for (int nt = 0; nt < NT; ++nt) {
+        acc[rt][nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(moe_as_bf16x8(wv[nt]), moe_as_bf16x8(av[rt]), acc[rt][nt], 0, 0, 0);
+        if (GLU) acc_up[rt][nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(moe_as_bf16x8(wu[nt]), moe_as_bf16x8(av[rt]), acc_up[rt][nt], 0, 0, 0);
+      }
   }
-  if (col >= rows) return;
 #pragma unroll
-  for (int nt = 0; nt < NT; ++nt)
+  for (int rt = 0; rt < RT; ++rt) {
+    if (16 * rt + col >= rows) continue;
 #pragma unroll
-    for (int r = 0; r < 4; ++r) {
-      const int o = o0 + 16 * nt + 4 * g + r;
-      if (o < F) out[(size_t)(first + col) * o_stride + o] = from_float<TO>(GLU ? moe_act(acc[nt][r], acc_up[nt][r], act) : acc[nt][r]);
-    }
+    for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        const int o = o0 + 16 * nt + 4 * g + r;
+        if (o < F)
+          out[(size_t)(first + 16 * rt + col) * o_stride + o] = from_float<TO>(GLU ? moe_act(acc[rt][nt][r], acc_up[rt][nt][r], act) : acc[rt][nt][r]);
+      }
+  }
 }
 
 // a [rows][K]; w [E][N][K] with N = F outputs, or with glu N = 2F: gate rows then up rows; out [P][F]
 extern "C" int lev_moe_linear(const void* a, long a_stride, const void* w, void* out, long o_stride, const int* tiles, const int* meta,
-                              const int* sorted, int max_tiles, int top, int gather, int K, int N, int glu, int act, int dtype, int out_dtype,
-                              int use_mfma, hipStream_t stream) {
+                              const int* sorted, int max_tiles, int tile_rows, int top, int gather, int K, int N, int glu, int act, int dtype,
+                              int out_dtype, int use_mfma, hipStream_t stream) {
   LEV_REQUIRE(a && w && out && tiles && meta && sorted, "experts: a tensor is missing");
   LEV_REQUIRE(K > 0 && N > 0 && (!glu || N % 2 == 0) && top > 0 && max_tiles >= 0, "experts: bad sizes K=%d N=%d", K, N);
   LEV_REQUIRE(act >= 0 && act <= LEV_ACT_LAST, "experts: unknown activation %d", act);
+  LEV_REQUIRE(tile_rows == MOE_TM || tile_rows == 4 * MOE_TM, "experts: tiles of %d rows (%d or %d)", tile_rows, MOE_TM, 4 * MOE_TM);
   LEV_REQUIRE(dtype == LEV_F32 || dtype == LEV_BF16, "experts: unknown dtype %d", dtype);
   LEV_REQUIRE(dtype == LEV_BF16 || out_dtype == LEV_F32, "experts: float32 inputs give float32 outputs");
   const int F = glu ? N / 2 : N;
@@ -249,16 +272,18 @@ extern "C" int lev_moe_linear(const void* a, long a_stride, const void* w, void*
   if (max_tiles == 0) return 0;
   if (dtype == LEV_BF16 && use_mfma && K % 8 == 0 && a_stride % 8 == 0 && ((uintptr_t)a & 15) == 0 && ((uintptr_t)w & 15) == 0) {
     // few tiles (a decoding step): one column tile a wave, so that the step has four times the waves
-    const int nt = max_tiles <= 64 ? 1 : 2;
+    const int nt = (max_tiles <= 64 && tile_rows == MOE_TM) ? 1 : 2;
     dim3 grid(max_tiles, (F + 64 * nt - 1) / (64 * nt));
+#define MOE_LAUNCH(TO, NTV, GLUV, RTV)                                                                                                            \
+  moe_linear_mfma_kernel<TO, NTV, GLUV, RTV><<<grid, 256, 0, stream>>>((const bf16_t*)a, a_stride, (const bf16_t*)w, (TO*)out, o_stride, tiles, meta, \
+                                                                       sorted, top, gather, K, N, F, act)
 #define MOE_CASE(TO, NTV)                                                                                                                        \
   do {                                                                                                                                           \
-    if (glu)                                                                                                                                     \
-      moe_linear_mfma_kernel<TO, NTV, true><<<grid, 256, 0, stream>>>((const bf16_t*)a, a_stride, (const bf16_t*)w, (TO*)out, o_stride, tiles, meta, \
-                                                                      sorted, top, gather, K, N, F, act);                                        \
-    else                                                                                                                                         \
-      moe_linear_mfma_kernel<TO, NTV, false><<<grid, 256, 0, stream>>>((const bf16_t*)a, a_stride, (const bf16_t*)w, (TO*)out, o_stride, tiles, meta, \
-                                                                       sorted, top, gather, K, N, F, act);                                       \
+    if (tile_rows == MOE_TM) {                                                                                                                   \
+      if (glu) MOE_LAUNCH(TO, NTV, true, 1); else MOE_LAUNCH(TO, NTV, false, 1);                                                                 \
+    } else {                                                                                                                                     \
+      if (glu) MOE_LAUNCH(TO, 2, true, 4); else MOE_LAUNCH(TO, 2, false, 4);                                                                     \
+    }                                                                                                                                            \
   } while (0)
     if (out_dtype == LEV_F32) {
       if (nt == 1) MOE_CASE(float, 1); else MOE_CASE(float, 2);
@@ -266,6 +291,7 @@ extern "C" int lev_moe_linear(const void* a, long a_stride, const void* w, void*
       if (nt == 1) MOE_CASE(bf16_t, 1); else MOE_CASE(bf16_t, 2);
     }
 #undef MOE_CASE
+#undef MOE_LAUNCH
     return lev_check_launch("moe_linear (matrix cores)");
   }
   dim3 grid(max_tiles, (F + 15) / 16);
@@ -285,17 +311,24 @@ extern "C" int lev_moe_linear(const void* a, long a_stride, const void* w, void*
 __global__ void __launch_bounds__(256)
 moe_combine_kernel(const float* __restrict__ expert_out, const int* __restrict__ pos_of, const float* __restrict__ weights, float* __restrict__ y,
                    int D, int top, int accumulate) {
+  __shared__ int pos_s[MOE_MAX_TOP];
+  __shared__ float w_s[MOE_MAX_TOP];
   const int t = blockIdx.x;
+  if (threadIdx.x < top) {
+    pos_s[threadIdx.x] = pos_of[(size_t)t * top + threadIdx.x];
+    w_s[threadIdx.x] = weights[(size_t)t * top + threadIdx.x];
+  }
+  __syncthreads();
   for (int d = threadIdx.x; d < D; d += 256) {
     float acc = accumulate ? y[(size_t)t * D + d] : 0.f;
-    for (int c = 0; c < top; ++c) acc = fmaf(weights[(size_t)t * top + c], expert_out[(size_t)pos_of[(size_t)t * top + c] * D + d], acc);
+    for (int c = 0; c < top; ++c) acc = fmaf(w_s[c], expert_out[(size_t)pos_s[c] * D + d], acc);
     y[(size_t)t * D + d] = acc;
   }
 }
 
 extern "C" int lev_moe_combine(const float* expert_out, const int* pos_of, const float* weights, float* y, int T, int D, int top, int accumulate,
                                hipStream_t stream) {
-  LEV_REQUIRE(expert_out && pos_of && weights && y && T >= 0 && D > 0 && top > 0, "experts: bad arguments of the weighted sum");
+  LEV_REQUIRE(expert_out && pos_of && weights && y && T >= 0 && D > 0 && top > 0 && top <= MOE_MAX_TOP, "experts: bad arguments of the weighted sum");
   if (T == 0) return 0;
   moe_combine_kernel<<<T, 256, 0, stream>>>(expert_out, pos_of, weights, y, D, top, accumulate);
   return lev_check_launch("moe_combine");

@@ -280,10 +280,12 @@ register_unit("core", ["errors.hip", "elementwise.hip", "layer_ops.hip", "gemm_s
     "lev_rotary_half": [_P, _L, _I, _I, _I, _I, _P, _P, _I, _I, _P],
     "lev_group_norm_step": [_P, _P, _P, _L, _I, _P, _F, _P, _P, _I, _P, _I, _I, _I, _F, _P],
     "lev_delta_rule": [_P] * 5 + [_L, _P, _L, _P, _P, _P, _P, _L, _I, _I, _I, _F, _F, _F, _I, _P],
+    "lev_delta_rule_scan": [_P] * 5 + [_L, _P, _L, _P, _P, _P, _P, _L, _P, _I, _I, _I, _I, _F, _F, _F, _I, _P],
+    "lev_delta_rule_scan_workspace": [_I, _I, _I],
     "lev_moe_route": [_P, _L, _P] + [_I] * 7 + [_P, _P, _P],
-    "lev_moe_max_tiles": [_I, _I],
-    "lev_moe_sort": [_P, _I, _I, _P, _P, _P, _P, _P],
-    "lev_moe_linear": [_P, _L, _P, _P, _L, _P, _P, _P] + [_I] * 10 + [_P],
+    "lev_moe_max_tiles": [_I, _I, _I],
+    "lev_moe_sort": [_P, _I, _I, _I, _P, _P, _P, _P, _P],
+    "lev_moe_linear": [_P, _L, _P, _P, _L, _P, _P, _P] + [_I] * 11 + [_P],
     "lev_moe_combine": [_P, _P, _P, _P, _I, _I, _I, _I, _P],
     "lev_block_linear": [_P, _L, _P, _P, _P, _L] + [_I] * 7 + [_P],
     "lev_block_linear_mfma": [_P, _L, _P, _P, _P, _L] + [_I] * 6 + [_P],

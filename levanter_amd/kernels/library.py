@@ -838,12 +838,14 @@ class HipKernels:
 
     # ---- a matrix state per head with decay and removal (generalized delta rule) ----------------
     def delta_rule(self, r, k, v, a_pre, g, w_pre, norm_weight, state, token_slots, out, n_heads: int, head_dim: int, norm_eps: float,
-                   key_eps: float, sharpness: float) -> None:
+                   key_eps: float, sharpness: float, max_runs: Optional[int] = None) -> None:
         """Per head, along each request's tokens, in 32-bit: ``u = k / sqrt(sum(k^2) + key_eps)``, ``w = exp(-sharpness *
         sigmoid(w_pre))``, ``a = sigmoid(a_pre)``, ``S <- diag(w) S - (a * u)(u^T S) + k v^T`` (both terms read the old ``S``),
         ``o = S^T r``, ``out = o / sqrt(mean(o^2) + norm_eps) * norm_weight * sigmoid(g)``. ``r, k, v, a_pre, g``: ``[T, H*d]``
         views of one row stride in the compute dtype; ``w_pre`` float32 ``[T, H*d]``; ``state`` float32 ``[slots, H, d, d]``
-        (key channel, value channel), read and stored; ``token_slots`` int32 ``[T]`` (-1: a token of nobody, zeros)."""
+        (key channel, value channel), read and stored; ``token_slots`` int32 ``[T]`` (-1: a token of nobody, zeros). ``max_runs``: the
+        step has at most this many runs of consecutive tokens of one slot; given, and smaller than T, the step takes the path for
+        prompts (the vectors of all tokens in parallel, then the walk along each run, then norm and gate in parallel)."""
         _dev(r, k, v, a_pre, g, w_pre, norm_weight, state, token_slots, out)
         T, C = r.shape
         dt = r.dtype
@@ -856,6 +858,12 @@ class HipKernels:
         _req(state.dtype == torch.float32 and state.is_contiguous() and tuple(state.shape[1:]) == (n_heads, head_dim, head_dim), "delta_rule: state must be float32 [slots, heads, d, d]")
         _req(token_slots.dtype == torch.int32 and token_slots.numel() == T, "delta_rule: one int32 slot per token")
         _req(out.dtype == dt and tuple(out.shape) == (T, C), "delta_rule: out must be [T, heads*head_dim] of the compute dtype")
+        if max_runs is not None and max_runs < T:
+            ws = torch.empty(self.lib.lev_delta_rule_scan_workspace(T, n_heads, head_dim) // 4, dtype=torch.float32, device=r.device)
+            self._check(self.lib.lev_delta_rule_scan(_ptr(r), _ptr(k), _ptr(v), _ptr(a_pre), _ptr(g), stride, _ptr(w_pre), _rows(w_pre, "delta_rule: w_pre"),
+                                                     _ptr(norm_weight), _ptr(state), _ptr(token_slots), _ptr(out), _rows(out, "delta_rule: out"), _ptr(ws), T,
+                                                     int(max_runs), n_heads, head_dim, float(norm_eps), float(key_eps), float(sharpness), _DT[dt], self._s()))
+            return
         self._check(self.lib.lev_delta_rule(_ptr(r), _ptr(k), _ptr(v), _ptr(a_pre), _ptr(g), stride, _ptr(w_pre), _rows(w_pre, "delta_rule: w_pre"),
                                             _ptr(norm_weight), _ptr(state), _ptr(token_slots), _ptr(out), _rows(out, "delta_rule: out"), T, n_heads,
                                             head_dim, float(norm_eps), float(key_eps), float(sharpness), _DT[dt], self._s()))
@@ -875,21 +883,27 @@ class HipKernels:
         self._check(self.lib.lev_moe_route(_ptr(z), _rows(z, "experts: z"), _ptr(correction), T, E, int(n_groups), int(keep), int(group_top), top,
                                            int(renormalize), _ptr(chosen), _ptr(weights), self._s()))
 
-    def moe_max_tiles(self, pairs: int, n_experts: int) -> int:
-        return int(self.lib.lev_moe_max_tiles(int(pairs), int(n_experts)))
+    @staticmethod
+    def moe_tile_rows(pairs: int, n_experts: int) -> int:
+        """Rows of a tile of the experts' products: 64 where an expert has 32 rows or more on average, else 16."""
+        return 64 if pairs >= 32 * n_experts else 16
 
-    def moe_sort(self, chosen, n_experts: int, sorted_pairs, pos_of, tiles, meta) -> None:
+    def moe_max_tiles(self, pairs: int, n_experts: int, tile_rows: int = 16) -> int:
+        return int(self.lib.lev_moe_max_tiles(int(pairs), int(n_experts), int(tile_rows)))
+
+    def moe_sort(self, chosen, n_experts: int, sorted_pairs, pos_of, tiles, meta, tile_rows: int = 16) -> None:
         """The (token, choice) pairs of ``chosen`` ordered by expert: ``sorted_pairs[pos]`` the pair at place ``pos``, ``pos_of`` its
-        inverse, ``tiles`` int32 ``[max_tiles, 3]`` (expert, first place, rows) covering every expert's stretch, ``meta[0]`` their
-        number. Everything stays on the device."""
+        inverse, ``tiles`` int32 ``[max_tiles, 3]`` (expert, first place, rows <= ``tile_rows``) covering every expert's stretch,
+        ``meta[0]`` their number. Everything stays on the device."""
         _dev(chosen, sorted_pairs, pos_of, tiles, meta)
         P = chosen.numel()
         for t in (chosen, sorted_pairs, pos_of, tiles, meta):
             _req(t.dtype == torch.int32 and t.is_contiguous(), "experts: int32 tables")
-        _req(sorted_pairs.numel() >= P and pos_of.numel() >= P and tiles.numel() >= 3 * self.moe_max_tiles(P, n_experts) and meta.numel() >= 1, "experts: tables too small")
-        self._check(self.lib.lev_moe_sort(_ptr(chosen), P, int(n_experts), _ptr(sorted_pairs), _ptr(pos_of), _ptr(tiles), _ptr(meta), self._s()))
+        _req(sorted_pairs.numel() >= P and pos_of.numel() >= P and tiles.numel() >= 3 * self.moe_max_tiles(P, n_experts, tile_rows) and meta.numel() >= 1, "experts: tables too small")
+        self._check(self.lib.lev_moe_sort(_ptr(chosen), P, int(n_experts), int(tile_rows), _ptr(sorted_pairs), _ptr(pos_of), _ptr(tiles), _ptr(meta), self._s()))
 
-    def moe_linear(self, a, w, out, tiles, meta, sorted_pairs, *, top: int, gather: bool, glu: bool = False, activation: str = "none") -> None:
+    def moe_linear(self, a, w, out, tiles, meta, sorted_pairs, *, top: int, gather: bool, glu: bool = False, activation: str = "none",
+                   tile_rows: int = 16) -> None:
         """For every tile of ``moe_sort``: ``out[pos] = w[expert] a[row(pos)]``, ``row(pos)`` the pair's token (``gather``) or
         ``pos`` itself. ``w`` ``[E, N, K]``; with ``glu`` N = 2F, gate rows then up rows, and ``out[pos][f] = act(gate_f) * up_f``."""
         _dev(a, w, out, tiles, meta, sorted_pairs)
@@ -899,7 +913,7 @@ class HipKernels:
         _req(out.dim() == 2 and out.shape[1] == F_ and out.dtype in _DT and (a.dtype == torch.bfloat16 or out.dtype == torch.float32), "experts: bad output")
         max_tiles = tiles.numel() // 3
         self._check(self.lib.lev_moe_linear(_ptr(a), _rows(a, "experts: a"), _ptr(w), _ptr(out), _rows(out, "experts: out"), _ptr(tiles), _ptr(meta),
-                                            _ptr(sorted_pairs), max_tiles, int(top), int(gather), K, N, int(glu), ACTIVATIONS[activation], _DT[a.dtype],
+                                            _ptr(sorted_pairs), max_tiles, int(tile_rows), int(top), int(gather), K, N, int(glu), ACTIVATIONS[activation], _DT[a.dtype],
                                             _DT[out.dtype], int(self.use_mfma), self._s()))
 
     def moe_combine(self, expert_out, pos_of, weights, y, accumulate: bool = False) -> None:

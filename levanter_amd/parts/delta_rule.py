@@ -95,5 +95,7 @@ class GeneralDeltaRule(Mixer):
         C, Cp = self.channels, self.part
         r, k, v, rem, g = (p[:, i * Cp:i * Cp + C] for i in range(5))
         w_pre = self.decay_up(self.decay_down(h, ctx, activation="tanh"), ctx, out_dtype=torch.float32)
+        # a step with prompt portions has fewer runs than tokens (at most one per request of the step): the path for prompts
+        max_runs = int(ctx.seq_slots.numel()) if ctx.attention.n_prefill_tiles else None
         K.delta_rule(r, k, v, rem, g, w_pre, self.norm_weight, unit.state, ctx.token_slots, a, self.n_heads, self.head_dim, self.norm_eps,
-                     self.key_eps, self.sharpness)
+                     self.key_eps, self.sharpness, max_runs=max_runs)

@@ -89,11 +89,12 @@ class RoutedExperts(FeedForward):
         weights = torch.empty((T, top), dtype=torch.float32, device=dev)
         K.moe_route(z, self.correction, chosen, weights, n_groups=self.n_groups, keep=self.keep, group_top=self.group_top, renormalize=self.renormalize)
         P = T * top
-        tables = torch.empty(2 * P + 3 * K.moe_max_tiles(P, E) + 1, dtype=torch.int32, device=dev)
+        rows = K.moe_tile_rows(P, E)  # prompts: four row tiles on every weight fragment a wave loads
+        tables = torch.empty(2 * P + 3 * K.moe_max_tiles(P, E, rows) + 1, dtype=torch.int32, device=dev)
         sorted_pairs, pos_of, meta, tiles = tables[:P], tables[P:2 * P], tables[2 * P:2 * P + 1], tables[2 * P + 1:]
-        K.moe_sort(chosen, E, sorted_pairs, pos_of, tiles, meta)
+        K.moe_sort(chosen, E, sorted_pairs, pos_of, tiles, meta, tile_rows=rows)
         inner = ctx.empty(P, self.inner_padded)
-        K.moe_linear(h, self.w_in, inner, tiles, meta, sorted_pairs, top=top, gather=True, glu=True, activation=self.activation)
+        K.moe_linear(h, self.w_in, inner, tiles, meta, sorted_pairs, top=top, gather=True, glu=True, activation=self.activation, tile_rows=rows)
         expert_out = ctx.empty(P, self.dim, torch.float32)
-        K.moe_linear(inner, self.w_down, expert_out, tiles, meta, sorted_pairs, top=top, gather=False)
+        K.moe_linear(inner, self.w_down, expert_out, tiles, meta, sorted_pairs, top=top, gather=False, tile_rows=rows)
         K.moe_combine(expert_out, pos_of, weights, y, accumulate=accumulate)

@@ -230,7 +230,7 @@ class EmulatedKernels:
         v[:, :, offset + n:offset + 2 * n] = (hi * cos + lo * sin).to(x.dtype)
 
     # ---- generalized delta rule
-    def delta_rule(self, r, k, v, a_pre, g, w_pre, norm_weight, state, token_slots, out, n_heads, head_dim, norm_eps, key_eps, sharpness) -> None:
+    def delta_rule(self, r, k, v, a_pre, g, w_pre, norm_weight, state, token_slots, out, n_heads, head_dim, norm_eps, key_eps, sharpness, max_runs=None) -> None:
         T, H, d = r.shape[0], n_heads, head_dim
         nw = norm_weight.view(H, d)
         for t in range(T):
@@ -269,12 +269,14 @@ class EmulatedKernels:
             wt = s[t][order]
             weights[t] = wt / wt.sum() if renormalize else wt
 
-    TILE_ROWS = 16
+    @staticmethod
+    def moe_tile_rows(pairs, n_experts) -> int:
+        return 64 if pairs >= 32 * n_experts else 16
 
-    def moe_max_tiles(self, pairs, n_experts) -> int:
-        return pairs // self.TILE_ROWS + n_experts + 1
+    def moe_max_tiles(self, pairs, n_experts, tile_rows=16) -> int:
+        return pairs // tile_rows + n_experts + 1
 
-    def moe_sort(self, chosen, n_experts, sorted_pairs, pos_of, tiles, meta) -> None:
+    def moe_sort(self, chosen, n_experts, sorted_pairs, pos_of, tiles, meta, tile_rows=16) -> None:
         flat = chosen.reshape(-1).long()
         order = torch.sort(flat, stable=True).indices
         P = flat.numel()
@@ -284,13 +286,13 @@ class EmulatedKernels:
         n, at = 0, 0
         for e in range(n_experts):
             count = int((flat == e).sum())
-            for i in range(0, count, self.TILE_ROWS):
-                tl[n] = torch.tensor([e, at + i, min(self.TILE_ROWS, count - i)], dtype=torch.int32)
+            for i in range(0, count, tile_rows):
+                tl[n] = torch.tensor([e, at + i, min(tile_rows, count - i)], dtype=torch.int32)
                 n += 1
             at += count
         meta[0] = n
 
-    def moe_linear(self, a, w, out, tiles, meta, sorted_pairs, *, top, gather, glu=False, activation="none") -> None:
+    def moe_linear(self, a, w, out, tiles, meta, sorted_pairs, *, top, gather, glu=False, activation="none", tile_rows=16) -> None:
         tl = tiles.view(-1, 3)
         F_ = out.shape[1]
         for i in range(int(meta[0])):

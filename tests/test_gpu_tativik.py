@@ -152,8 +152,9 @@ def plain_delta(p, w_pre, nw, H, d, eps, state=None):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("H,d", [(2, 16), (3, 10), (1, 64), (4, 48), (2, 128), (1, 1)])
-def test_the_delta_rule_carries_its_state_through_any_cutting(dtype, H, d):
+@pytest.mark.parametrize("H,d", [(2, 16), (3, 10), (1, 64), (4, 48), (2, 128), (1, 1), (1, 200)])
+@pytest.mark.parametrize("prompt_path", [False, True])
+def test_the_delta_rule_carries_its_state_through_any_cutting(dtype, H, d, prompt_path):
     """Two requests and a token of nobody, cut into steps of several sizes down to one token: outputs and the slots' states are
     the plain scan's; the slots of others stay as they are."""
     g = torch.Generator().manual_seed(H * 100 + d)
@@ -182,7 +183,7 @@ def test_the_delta_rule_carries_its_state_through_any_cutting(dtype, H, d):
         p = dev(torch.cat(rows), dtype)
         out = torch.full((p.shape[0], C), float("nan"), dtype=dtype, device=DEV)
         K().delta_rule(*(p[:, i * C:(i + 1) * C] for i in range(5)), dev(torch.cat(wrows)), dev(nw), state, torch.tensor(slots, dtype=torch.int32, device=DEV),
-                       out, H, d, eps, P.UNIT_KEY_EPS, P.DECAY_SHARPNESS)
+                       out, H, d, eps, P.UNIT_KEY_EPS, P.DECAY_SHARPNESS, max_runs=len(sizes) if prompt_path else None)
         t = 0
         for s, n in sizes:
             if s < 0:
@@ -196,6 +197,33 @@ def test_the_delta_rule_carries_its_state_through_any_cutting(dtype, H, d):
         torch.testing.assert_close(torch.cat(got[s]), want[s][0], **tol(dtype, f32=2e-4, bf16=3e-2))
         torch.testing.assert_close(state[s].cpu().double(), want[s][1], rtol=2e-4, atol=2e-4)
     assert bool((state[1] == 7.0).all()) and bool(state[3].isnan().all())
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("H,d", [(2, 16), (3, 10), (2, 128), (1, 256)])
+def test_the_prompt_path_of_the_delta_rule_on_long_runs_beside_single_tokens(dtype, H, d):
+    """Runs of 300 and 150 tokens, two single tokens and a token of nobody in one step, from states that are not zero."""
+    g = torch.Generator().manual_seed(d)
+    C = H * d
+    lens = [(0, 300), (3, 1), (-1, 1), (1, 150), (2, 1)]
+    state0 = torch.randn(4, H, d, d, generator=g) * 0.3
+    state = state0.to(DEV)
+    rows, wrows, slots, want = [], [], [], []
+    nw = 1 + 0.2 * torch.randn(C, generator=g)
+    for s, n in lens:
+        p, w_pre, _ = delta_inputs(n, H, d, g, dtype)
+        rows.append(p)
+        wrows.append(w_pre)
+        slots += [s] * n
+        want.append(plain_delta(p, w_pre, nw, H, d, 1e-5, state0[s].double()) if s >= 0 else (torch.zeros(n, C, dtype=torch.float64), None))
+    p = dev(torch.cat(rows), dtype)
+    out = torch.full((p.shape[0], C), float("nan"), dtype=dtype, device=DEV)
+    K().delta_rule(*(p[:, i * C:(i + 1) * C] for i in range(5)), dev(torch.cat(wrows)), dev(nw), state, torch.tensor(slots, dtype=torch.int32, device=DEV), out,
+                   H, d, 1e-5, P.UNIT_KEY_EPS, P.DECAY_SHARPNESS, max_runs=7)
+    torch.testing.assert_close(out.cpu().double(), torch.cat([w[0] for w in want]), **tol(dtype, f32=5e-4, bf16=3e-2))
+    for (s, n), w in zip(lens, want):
+        if s >= 0:
+            torch.testing.assert_close(state[s].cpu().double(), w[1], rtol=5e-4, atol=5e-4)
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
@@ -245,7 +273,8 @@ def test_the_router(T, E, G, keep, top):
 
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("T,D,F,E,top", [(37, 64, 24, 8, 2), (1, 32, 8, 2, 1), (300, 96, 48, 12, 3), (5, 40, 13, 5, 2), (64, 256, 96, 4, 4), (9, 128, 200, 3, 1)])
-def test_the_experts_products_over_tokens_sorted_by_expert(dtype, T, D, F, E, top):
+@pytest.mark.parametrize("rows", [16, 64])
+def test_the_experts_products_over_tokens_sorted_by_expert(dtype, T, D, F, E, top, rows):
     g = torch.Generator().manual_seed(T + F)
     h = bfn(torch.randn(T, D, generator=g))
     W = {}
@@ -265,9 +294,9 @@ def test_the_experts_products_over_tokens_sorted_by_expert(dtype, T, D, F, E, to
         w_in[e, :F], w_in[e, Fp:Fp + F], w_down[e, :, :F] = W[f"m.e{e}.gate"], W[f"m.e{e}.up"], W[f"m.e{e}.down"]
     kern = K()
     Pn = T * top
-    tables = torch.full((2 * Pn + 3 * kern.moe_max_tiles(Pn, E) + 1,), -7, dtype=torch.int32, device=DEV)
+    tables = torch.full((2 * Pn + 3 * kern.moe_max_tiles(Pn, E, rows) + 1,), -7, dtype=torch.int32, device=DEV)
     sorted_pairs, pos_of, meta, tiles = tables[:Pn], tables[Pn:2 * Pn], tables[2 * Pn:2 * Pn + 1], tables[2 * Pn + 1:]
-    kern.moe_sort(chosen.to(DEV), E, sorted_pairs, pos_of, tiles, meta)
+    kern.moe_sort(chosen.to(DEV), E, sorted_pairs, pos_of, tiles, meta, tile_rows=rows)
     sp, po = sorted_pairs.cpu().long(), pos_of.cpu().long()
     assert sorted(sp.tolist()) == list(range(Pn)) and torch.equal(sp[po], torch.arange(Pn))
     flat = chosen.reshape(-1).long()
@@ -275,11 +304,11 @@ def test_the_experts_products_over_tokens_sorted_by_expert(dtype, T, D, F, E, to
     n_tiles = int(meta[0])
     tl = tiles.cpu().view(-1, 3)[:n_tiles]
     covered = torch.cat([torch.arange(int(f), int(f) + int(n)) for _, f, n in tl])
-    assert torch.equal(covered, torch.arange(Pn)) and all(bool((flat[sp][int(f):int(f) + int(n)] == int(e)).all()) and 0 < int(n) <= 16 for e, f, n in tl)
+    assert torch.equal(covered, torch.arange(Pn)) and all(bool((flat[sp][int(f):int(f) + int(n)] == int(e)).all()) and 0 < int(n) <= rows for e, f, n in tl)
     inner = torch.full((Pn, Fp), float("nan"), dtype=dtype, device=DEV)
-    kern.moe_linear(dev(h, dtype), dev(w_in, dtype), inner, tiles, meta, sorted_pairs, top=top, gather=True, glu=True, activation="silu")
+    kern.moe_linear(dev(h, dtype), dev(w_in, dtype), inner, tiles, meta, sorted_pairs, top=top, gather=True, glu=True, activation="silu", tile_rows=rows)
     eo = torch.full((Pn, D), float("nan"), dtype=torch.float32, device=DEV)
-    kern.moe_linear(inner, dev(w_down, dtype), eo, tiles, meta, sorted_pairs, top=top, gather=False)
+    kern.moe_linear(inner, dev(w_down, dtype), eo, tiles, meta, sorted_pairs, top=top, gather=False, tile_rows=rows)
     y = torch.full((T, D), float("nan"), dtype=torch.float32, device=DEV)
     kern.moe_combine(eo, pos_of, dev(weights), y)
     want = torch.zeros(T, D, dtype=torch.float64)

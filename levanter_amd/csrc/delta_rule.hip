@@ -112,8 +112,8 @@ extern "C" int lev_delta_rule(const void* r, const void* k, const void* v, const
 // ---- runs of many tokens (prompt portions) --------------------------------------------------------------------------------
 // The kernel above walks a run with one thread per state column and all of a token's work between barriers. For prompts the
 // work is split in three: (1) per token and head, in parallel over the step: u, w, a * u, k, r as float32 vectors; (2) the
-// walk itself, one workgroup per (run, head) of DMAX columns x P parts: thread (part, j) keeps the key channels of its part of
-// column j in registers, a token's vectors are staged through LDS one token ahead, the only sum across threads inside the
+// walk itself, one workgroup per (run, head, 32 state columns) of 32 columns x P parts: thread (part, j) keeps the key channels of
+// its part of column j in registers, a token's vectors are staged through LDS one token ahead, the only sum across threads inside the
 // loop is u^T S (P partial sums through LDS), and the partial sums of o = S^T r go to scratch memory; (3) per token and head,
 // in parallel: o from its parts, the head's norm, the weight and the gate. Two barriers a token.
 template <typename T, int DMAX>
@@ -139,17 +139,18 @@ delta_prepare_kernel(const T* __restrict__ r, const T* __restrict__ k, const T* 
   o[4 * d] = rf;
 }
 
+#define DELTA_CB 32  // state columns of a workgroup of the walk: columns never meet, so a head's columns are split over workgroups
 template <typename T, int DMAX, int P>
-__global__ void __launch_bounds__(DMAX * P)
+__global__ void __launch_bounds__(DELTA_CB * P)
 delta_scan_kernel(const float* __restrict__ vec, const T* __restrict__ v, long stride, float* __restrict__ state, const int* __restrict__ token_slots,
                   float* __restrict__ part_o /*[Tn][H][P][d]*/, int Tn, int H, int d) {
-  constexpr int NT = DMAX * P, IP = DMAX / P;
+  constexpr int NT = DELTA_CB * P, IP = DMAX / P;
   __shared__ float s_vec[2][5][DMAX];
-  __shared__ float s_pu[2][P][DMAX];
+  __shared__ float s_pu[2][P][DELTA_CB];
   __shared__ int s_count[NT];
   __shared__ int s_start;
   const int run = blockIdx.x, h = blockIdx.y, tid = threadIdx.x;
-  const int part = tid / DMAX, j = tid - part * DMAX;
+  const int part = tid / DELTA_CB, jj = tid - part * DELTA_CB, j = blockIdx.z * DELTA_CB + jj;
   // the run-th run of the step: a token starts one if it has a slot and the token before it has another. Each thread counts
   // the starts of its stretch of tokens; the thread whose stretch holds the run-th one finds it.
   const int per = (Tn + NT - 1) / NT, lo = tid * per, hi = min(Tn, lo + per);
@@ -208,11 +209,11 @@ delta_scan_kernel(const float* __restrict__ vec, const T* __restrict__ v, long s
     float pu = 0.f;
 #pragma unroll
     for (int ii = 0; ii < IP; ++ii) pu = fmaf(su[ii], S[ii], pu);
-    s_pu[buf][part][j] = pu;
+    s_pu[buf][part][jj] = pu;
     __syncthreads();
     float uS = 0.f;
 #pragma unroll
-    for (int q = 0; q < P; ++q) uS += s_pu[buf][q][j];
+    for (int q = 0; q < P; ++q) uS += s_pu[buf][q][jj];
     float o = 0.f;
 #pragma unroll
     for (int ii = 0; ii < IP; ++ii) {
@@ -274,12 +275,12 @@ extern "C" int lev_delta_rule_scan(const void* r, const void* k, const void* v, 
   float* vec = workspace;
   float* part_o = workspace + (size_t)Tn * H * 5 * d;
   const int P = delta_parts(d);
-  dim3 grid(Tn, H), runs(max_runs > 0 ? max_runs : 1, H);
+  dim3 grid(Tn, H), runs(max_runs > 0 ? max_runs : 1, H, (d + DELTA_CB - 1) / DELTA_CB);
 #define DS_CASE(TT, DM, PP)                                                                                                                        \
   do {                                                                                                                                             \
     delta_prepare_kernel<TT, DM><<<grid, DM, 0, stream>>>((const TT*)r, (const TT*)k, (const TT*)a_pre, stride, w_pre, w_stride, vec, H, d, key_eps,  \
                                                           sharpness);                                                                              \
-    delta_scan_kernel<TT, DM, PP><<<runs, DM * PP, 0, stream>>>(vec, (const TT*)v, stride, state, token_slots, part_o, Tn, H, d);                     \
+    delta_scan_kernel<TT, DM, PP><<<runs, DELTA_CB * PP, 0, stream>>>(vec, (const TT*)v, stride, state, token_slots, part_o, Tn, H, d);                     \
     delta_finish_kernel<TT, DM><<<grid, DM, 0, stream>>>(part_o, PP, (const TT*)g, stride, norm_w, token_slots, (TT*)out, o_stride, H, d, norm_eps); \
   } while (0)
   if (dtype == LEV_F32) {

@@ -220,6 +220,7 @@ moe_linear_mfma_kernel(const bf16_t* __restrict__ a, long a_stride, const bf16_t
   for (int rt = 0; rt < RT; ++rt)
 #pragma unroll
     for (int nt = 0; nt < NT; ++nt) acc[rt][nt] = acc_up[rt][nt] = moe_f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll 4
   for (int k0 = 0; k0 < K; k0 += 32) {
     const int kk = k0 + 8 * g, kc = min(kk, K - 8);  // loads stand under no condition; a chunk beyond the row counts as zeros
     const uint32_t keep = kk < K ? 0xffffffffu : 0u;
@@ -257,6 +258,60 @@ moe_linear_mfma_kernel(const bf16_t* __restrict__ a, long a_stride, const bf16_t
   }
 }
 
+// Few tiles (a step of single tokens): the products are bound by reading the chosen experts' weights, and a tile's 16 rows give
+// the chip too few waves. A workgroup of MOE_KS waves owns one tile of 16 rows and 16 outputs; its waves split K, every wave has
+// all loads of its share in flight, and the partial sums are added through LDS in wave order.
+#define MOE_KS 8
+template <typename TO, bool GLU>
+__global__ void __launch_bounds__(64 * MOE_KS)
+moe_linear_splitk_kernel(const bf16_t* __restrict__ a, long a_stride, const bf16_t* __restrict__ w, TO* __restrict__ out, long o_stride,
+                         const int* __restrict__ tiles, const int* __restrict__ meta, const int* __restrict__ sorted, int top, int gather,
+                         int K, int N, int F, int act) {
+  __shared__ float part[MOE_KS][2][4][64];
+  const int tile = blockIdx.x;
+  if (tile >= meta[0]) return;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, col = lane & 15, g = lane >> 4;
+  const int o0 = blockIdx.y * 16;
+  const int e = tiles[3 * tile], first = tiles[3 * tile + 1], rows = tiles[3 * tile + 2];
+  const int pos = first + min(col, rows - 1);  // rows beyond the tile: read again, never stored
+  const bf16_t* ar = a + (size_t)(gather ? sorted[pos] / top : pos) * a_stride;
+  const bf16_t* wr = w + (size_t)e * N * K + (size_t)min(o0 + col, F - 1) * K;
+  const int share = ((K + MOE_KS * 32 - 1) / (MOE_KS * 32)) * 32;  // k steps of 32 a wave
+  const int k_lo = wave * share, k_hi = min(K, k_lo + share);
+  moe_f32x4 acc = moe_f32x4{0.f, 0.f, 0.f, 0.f}, acc_up = acc;
+#pragma unroll 4
+  for (int k0 = k_lo; k0 < k_hi; k0 += 32) {
+    const int kk = k0 + 8 * g, kc = min(kk, K - 8);  // loads stand under no condition; a chunk beyond the row counts as zeros
+    const uint32_t keep = kk < K ? 0xffffffffu : 0u;
+    const moe_u32x4 x = *reinterpret_cast<const moe_u32x4*>(ar + kc);
+    const moe_u32x4 av = moe_u32x4{x[0] & keep, x[1] & keep, x[2] & keep, x[3] & keep};
+    const moe_u32x4 wv = *reinterpret_cast<const moe_u32x4*>(wr + kc);
+    acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(moe_as_bf16x8(wv), moe_as_bf16x8(av), acc, 0, 0, 0);
+    if (GLU) {
+      const moe_u32x4 wu = *reinterpret_cast<const moe_u32x4*>(wr + (size_t)F * K + kc);
+      acc_up = __builtin_amdgcn_mfma_f32_16x16x32_bf16(moe_as_bf16x8(wu), moe_as_bf16x8(av), acc_up, 0, 0, 0);
+    }
+  }
+#pragma unroll
+  for (int r = 0; r < 4; ++r) {
+    part[wave][0][r][lane] = acc[r];
+    if (GLU) part[wave][1][r][lane] = acc_up[r];
+  }
+  __syncthreads();
+  if (wave != 0 || col >= rows) return;
+#pragma unroll
+  for (int r = 0; r < 4; ++r) {
+    float sum = 0.f, sum_up = 0.f;
+#pragma unroll
+    for (int q = 0; q < MOE_KS; ++q) {
+      sum += part[q][0][r][lane];
+      if (GLU) sum_up += part[q][1][r][lane];
+    }
+    const int o = o0 + 4 * g + r;
+    if (o < F) out[(size_t)(first + col) * o_stride + o] = from_float<TO>(GLU ? moe_act(sum, sum_up, act) : sum);
+  }
+}
+
 // a [rows][K]; w [E][N][K] with N = F outputs, or with glu N = 2F: gate rows then up rows; out [P][F]
 extern "C" int lev_moe_linear(const void* a, long a_stride, const void* w, void* out, long o_stride, const int* tiles, const int* meta,
                               const int* sorted, int max_tiles, int tile_rows, int top, int gather, int K, int N, int glu, int act, int dtype,
@@ -271,8 +326,23 @@ extern "C" int lev_moe_linear(const void* a, long a_stride, const void* w, void*
   LEV_REQUIRE(a_stride >= K && o_stride >= F, "experts: row strides are smaller than the rows");
   if (max_tiles == 0) return 0;
   if (dtype == LEV_BF16 && use_mfma && K % 8 == 0 && a_stride % 8 == 0 && ((uintptr_t)a & 15) == 0 && ((uintptr_t)w & 15) == 0) {
-    // few tiles (a decoding step): one column tile a wave, so that the step has four times the waves
-    const int nt = (max_tiles <= 64 && tile_rows == MOE_TM) ? 1 : 2;
+    if (tile_rows == MOE_TM && max_tiles <= 96) {  // a step of single tokens: K split over the waves of a workgroup
+      dim3 grid_k(max_tiles, (F + 15) / 16);
+#define MOE_SPLITK(TO)                                                                                                                           \
+  do {                                                                                                                                           \
+    if (glu)                                                                                                                                     \
+      moe_linear_splitk_kernel<TO, true><<<grid_k, 64 * MOE_KS, 0, stream>>>((const bf16_t*)a, a_stride, (const bf16_t*)w, (TO*)out, o_stride, tiles, \
+                                                                            meta, sorted, top, gather, K, N, F, act);                            \
+    else                                                                                                                                         \
+      moe_linear_splitk_kernel<TO, false><<<grid_k, 64 * MOE_KS, 0, stream>>>((const bf16_t*)a, a_stride, (const bf16_t*)w, (TO*)out, o_stride, tiles, \
+                                                                             meta, sorted, top, gather, K, N, F, act);                           \
+  } while (0)
+      if (out_dtype == LEV_F32) MOE_SPLITK(float); else MOE_SPLITK(bf16_t);
+#undef MOE_SPLITK
+      return lev_check_launch("moe_linear (matrix cores, K split)");
+    }
+    // few tiles: one column tile a wave, so that the step has four times the waves; tiles of 64 rows: four
+    const int nt = tile_rows != MOE_TM ? 4 : max_tiles <= 64 ? 1 : 2;
     dim3 grid(max_tiles, (F + 64 * nt - 1) / (64 * nt));
 #define MOE_LAUNCH(TO, NTV, GLUV, RTV)                                                                                                            \
   moe_linear_mfma_kernel<TO, NTV, GLUV, RTV><<<grid, 256, 0, stream>>>((const bf16_t*)a, a_stride, (const bf16_t*)w, (TO*)out, o_stride, tiles, meta, \
@@ -282,7 +352,7 @@ extern "C" int lev_moe_linear(const void* a, long a_stride, const void* w, void*
     if (tile_rows == MOE_TM) {                                                                                                                   \
       if (glu) MOE_LAUNCH(TO, NTV, true, 1); else MOE_LAUNCH(TO, NTV, false, 1);                                                                 \
     } else {                                                                                                                                     \
-      if (glu) MOE_LAUNCH(TO, 2, true, 4); else MOE_LAUNCH(TO, 2, false, 4);                                                                     \
+      if (glu) MOE_LAUNCH(TO, 4, true, 4); else MOE_LAUNCH(TO, 4, false, 4);                                                                     \
     }                                                                                                                                            \
   } while (0)
     if (out_dtype == LEV_F32) {

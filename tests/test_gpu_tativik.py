@@ -272,7 +272,7 @@ def test_the_router(T, E, G, keep, top):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("T,D,F,E,top", [(37, 64, 24, 8, 2), (1, 32, 8, 2, 1), (300, 96, 48, 12, 3), (5, 40, 13, 5, 2), (64, 256, 96, 4, 4), (9, 128, 200, 3, 1)])
+@pytest.mark.parametrize("T,D,F,E,top", [(37, 64, 24, 8, 2), (1, 32, 8, 2, 1), (300, 96, 48, 12, 3), (5, 40, 13, 5, 2), (64, 256, 96, 4, 4), (9, 128, 200, 3, 1), (700, 64, 24, 40, 2)])
 @pytest.mark.parametrize("rows", [16, 64])
 def test_the_experts_products_over_tokens_sorted_by_expert(dtype, T, D, F, E, top, rows):
     g = torch.Generator().manual_seed(T + F)

@@ -113,8 +113,8 @@ extern "C" int lev_delta_rule(const void* r, const void* k, const void* v, const
 // The kernel above walks a run with one thread per state column and all of a token's work between barriers. For prompts the
 // work is split in three: (1) per token and head, in parallel over the step: u, w, a * u, k, r as float32 vectors; (2) the
 // walk itself, one workgroup per (run, head, 32 state columns) of 32 columns x P parts: thread (part, j) keeps the key channels of
-// its part of column j in registers, a token's vectors are staged through LDS one token ahead, the only sum across threads inside the
-// loop is u^T S (P partial sums through LDS), and the partial sums of o = S^T r go to scratch memory; (3) per token and head,
+// its part of column j in registers, a token's vectors are staged through LDS a block of tokens ahead, the only sum across threads inside
+// the loop is u^T S (P partial sums through LDS), and the partial sums of o = S^T r go to scratch memory; (3) per token and head,
 // in parallel: o from its parts, the head's norm, the weight and the gate. Two barriers a token.
 template <typename T, int DMAX>
 __global__ void __launch_bounds__(DMAX)
@@ -144,8 +144,8 @@ template <typename T, int DMAX, int P>
 __global__ void __launch_bounds__(DELTA_CB * P)
 delta_scan_kernel(const float* __restrict__ vec, const T* __restrict__ v, long stride, float* __restrict__ state, const int* __restrict__ token_slots,
                   float* __restrict__ part_o /*[Tn][H][P][d]*/, int Tn, int H, int d) {
-  constexpr int NT = DELTA_CB * P, IP = DMAX / P;
-  __shared__ float s_vec[2][5][DMAX];
+  constexpr int NT = DELTA_CB * P, IP = DMAX / P, TB = 1024 / DMAX;  // tokens whose vectors are staged together
+  __shared__ float s_vec[2][TB][5][DMAX];
   __shared__ float s_pu[2][P][DELTA_CB];
   __shared__ int s_count[NT];
   __shared__ int s_start;
@@ -171,8 +171,19 @@ delta_scan_kernel(const float* __restrict__ vec, const T* __restrict__ v, long s
   }
   __syncthreads();
   const int t0 = s_start;
+  __syncthreads();  // every thread has read it before it is used again below
   if (t0 < 0) return;  // the step has fewer runs (the whole workgroup)
   const int slot = token_slots[t0];
+  // where the run ends: the first later token of another slot (the walk itself then reads no table)
+  if (tid == 0) s_start = Tn;
+  __syncthreads();
+  for (int t = max(lo, t0 + 1); t < hi; ++t)
+    if (token_slots[t] != slot) {
+      atomicMin(&s_start, t);
+      break;
+    }
+  __syncthreads();
+  const int t_end = s_start;
   const bool live = j < d;
   float S[IP];
   float* sp = state + ((size_t)slot * H + h) * d * d + (live ? j : 0);
@@ -182,52 +193,66 @@ delta_scan_kernel(const float* __restrict__ vec, const T* __restrict__ v, long s
     S[ii] = (i < d && live) ? sp[(size_t)i * d] : 0.f;
   }
   const size_t col = (size_t)h * d + (live ? j : 0);
-  // stage the first token's vectors; elements beyond d are zeros
-  for (int idx = tid; idx < 5 * DMAX; idx += NT) {
-    const int which = idx / DMAX, i = idx - which * DMAX;
-    s_vec[0][which][i] = i < d ? vec[((size_t)t0 * H + h) * 5 * d + (size_t)which * d + i] : 0.f;
+  // The vectors of TB tokens at a time go through LDS: a block's loads are asked for when the block before it starts, so they
+  // have TB steps of the walk to arrive (asked for one token ahead, every step waited for its own loads' way through the
+  // memory). Elements beyond d are zeros.
+  constexpr int BLOCK = TB * 5 * DMAX, PER = (BLOCK + NT - 1) / NT;
+  float vcur[TB];
+  for (int idx = tid; idx < BLOCK; idx += NT) {
+    const int tt = idx / (5 * DMAX), rem = idx - tt * (5 * DMAX), which = rem / DMAX, i = rem - which * DMAX;
+    const int t = min(t0 + tt, Tn - 1);
+    s_vec[0][tt][which][i] = i < d ? vec[((size_t)t * H + h) * 5 * d + (size_t)which * d + i] : 0.f;
   }
-  float vf = live ? to_float<T>(v[(size_t)t0 * stride + col]) : 0.f;
+#pragma unroll
+  for (int tt = 0; tt < TB; ++tt) vcur[tt] = live ? to_float<T>(v[(size_t)min(t0 + tt, Tn - 1) * stride + col]) : 0.f;
   int buf = 0;
-  for (int t = t0;; ++t) {
-    const int tn = min(t + 1, Tn - 1);
-    const bool more = t + 1 < Tn && token_slots[tn] == slot;
-    // the next token's vectors and value are asked for now and put into LDS when this token is done
-    float nxt[(5 * DMAX + NT - 1) / NT];
+  for (int tb = t0; tb < t_end; tb += TB) {
+    float nxt[PER], vnext[TB];
+    const int nb = tb + TB;
 #pragma unroll
-    for (int n = 0; n < (5 * DMAX + NT - 1) / NT; ++n) {
-      const int idx = tid + n * NT, which = min(idx / DMAX, 4), i = idx - (idx / DMAX) * DMAX;
-      nxt[n] = vec[((size_t)tn * H + h) * 5 * d + (size_t)which * d + min(i, d - 1)];
+    for (int n = 0; n < PER; ++n) {
+      const int idx = min(tid + n * NT, BLOCK - 1);
+      const int tt = idx / (5 * DMAX), rem = idx - tt * (5 * DMAX), which = rem / DMAX, i = rem - which * DMAX;
+      nxt[n] = vec[((size_t)min(nb + tt, Tn - 1) * H + h) * 5 * d + (size_t)which * d + min(i, d - 1)];
     }
-    const float vn = to_float<T>(v[(size_t)tn * stride + col]);
-    __syncthreads();  // this token's vectors are in s_vec[buf]
-    const float* sw = s_vec[buf][0] + part * IP;
-    const float* sau = s_vec[buf][1] + part * IP;
-    const float* su = s_vec[buf][2] + part * IP;
-    const float* sk = s_vec[buf][3] + part * IP;
-    const float* sr = s_vec[buf][4] + part * IP;
-    float pu = 0.f;
 #pragma unroll
-    for (int ii = 0; ii < IP; ++ii) pu = fmaf(su[ii], S[ii], pu);
-    s_pu[buf][part][jj] = pu;
-    __syncthreads();
-    float uS = 0.f;
+    for (int tt = 0; tt < TB; ++tt) vnext[tt] = to_float<T>(v[(size_t)min(nb + tt, Tn - 1) * stride + col]);
 #pragma unroll
-    for (int q = 0; q < P; ++q) uS += s_pu[buf][q][jj];
-    float o = 0.f;
+    for (int tt = 0; tt < TB; ++tt) {
+      const int t = tb + tt;
+      if (t >= t_end) break;  // the whole workgroup
+      lds_barrier();  // the block's vectors are in s_vec[buf]; the loads in flight are the thread's own and are not waited for
+      const float* sw = s_vec[buf][tt][0] + part * IP;
+      const float* sau = s_vec[buf][tt][1] + part * IP;
+      const float* su = s_vec[buf][tt][2] + part * IP;
+      const float* sk = s_vec[buf][tt][3] + part * IP;
+      const float* sr = s_vec[buf][tt][4] + part * IP;
+      float pu = 0.f;
 #pragma unroll
-    for (int ii = 0; ii < IP; ++ii) {
-      S[ii] = fmaf(sk[ii], vf, fmaf(sw[ii], S[ii], -(sau[ii] * uS)));
-      o = fmaf(S[ii], sr[ii], o);
+      for (int ii = 0; ii < IP; ++ii) pu = fmaf(su[ii], S[ii], pu);
+      s_pu[tt & 1][part][jj] = pu;
+      lds_barrier();
+      float uS = 0.f;
+#pragma unroll
+      for (int q = 0; q < P; ++q) uS += s_pu[tt & 1][q][jj];
+      const float vf = vcur[tt];
+      float o = 0.f;
+#pragma unroll
+      for (int ii = 0; ii < IP; ++ii) {
+        S[ii] = fmaf(sk[ii], vf, fmaf(sw[ii], S[ii], -(sau[ii] * uS)));
+        o = fmaf(S[ii], sr[ii], o);
+      }
+      if (live) part_o[(((size_t)t * H + h) * P + part) * d + j] = o;
     }
-    if (live) part_o[(((size_t)t * H + h) * P + part) * d + j] = o;
-    if (!more) break;
+    if (nb >= t_end) break;
 #pragma unroll
-    for (int n = 0; n < (5 * DMAX + NT - 1) / NT; ++n) {
-      const int idx = tid + n * NT, which = idx / DMAX, i = idx - which * DMAX;
-      if (idx < 5 * DMAX) s_vec[buf ^ 1][which][i] = i < d ? nxt[n] : 0.f;
+    for (int n = 0; n < PER; ++n) {
+      const int idx = tid + n * NT;
+      const int tt = idx / (5 * DMAX), rem = idx - tt * (5 * DMAX), which = rem / DMAX, i = rem - which * DMAX;
+      if (idx < BLOCK) s_vec[buf ^ 1][tt][which][i] = i < d ? nxt[n] : 0.f;
     }
-    vf = live ? vn : 0.f;
+#pragma unroll
+    for (int tt = 0; tt < TB; ++tt) vcur[tt] = live ? vnext[tt] : 0.f;
     buf ^= 1;
   }
   if (live) {

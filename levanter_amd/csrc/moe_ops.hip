@@ -11,8 +11,9 @@
 //             fragment it loads).
 //   linear    for every tile: out[pos][o] = sum_k w[expert][o][k] a[row(pos)][k], row(pos) = the pair's token (gather) or pos
 //             itself; with glu the expert's matrix is [gate ; up] (2F rows) and out[pos][f] = act(gate_f) * up_f.
-//             bfloat16 on the matrix cores (16x16x32, both operands straight from global memory, as the block-diagonal
-//             product does), float32 in plain arithmetic. Workgroups beyond n_tiles return at once.
+//             bfloat16 on the matrix cores (16x16x32): few tiles of 16 rows with K split over a workgroup's waves, many with a
+//             wave per tile, tiles of 64 rows with both operands staged through LDS; float32 in plain arithmetic. Workgroups
+//             beyond n_tiles return at once.
 //   combine   y[t] = sum_c weight[t][c] * out[pos_of[t * top + c]], c in order, float32; with `accumulate` added to what y holds.
 #include "common.h"
 
@@ -312,6 +313,95 @@ moe_linear_splitk_kernel(const bf16_t* __restrict__ a, long a_stride, const bf16
   }
 }
 
+// Tiles of 64 rows (prompts): a workgroup of four waves owns a tile's 64 rows and 128 outputs (with glu: 128 of gate and the same
+// 128 of up); the rows' and the weights' k-steps of 32 go from global memory into registers one step ahead and from there into
+// LDS (two buffers, rows 40 elements apart so that the fragments' 16-byte reads spread over the banks), and every wave takes
+// its fragments from there: a weight or activation byte is fetched once a workgroup instead of once a wave.
+#define MOE_BN 128
+#define MOE_LD 40
+template <typename TO, bool GLU>
+__global__ void __launch_bounds__(256)
+moe_linear_tile_kernel(const bf16_t* __restrict__ a, long a_stride, const bf16_t* __restrict__ w, TO* __restrict__ out, long o_stride,
+                       const int* __restrict__ tiles, const int* __restrict__ meta, const int* __restrict__ sorted, int top, int gather,
+                       int K, int N, int F, int act) {
+  constexpr int WR = GLU ? 2 * MOE_BN : MOE_BN, WL = WR / 64;  // weight rows of a workgroup, loads of them per thread and k-step
+  __shared__ __attribute__((aligned(16))) bf16_t sa[2][64][MOE_LD];
+  __shared__ __attribute__((aligned(16))) bf16_t sw[2][WR][MOE_LD];
+  const int tile = blockIdx.x;
+  if (tile >= meta[0]) return;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, col = lane & 15, g = lane >> 4;
+  const int o0 = blockIdx.y * MOE_BN;
+  const int e = tiles[3 * tile], first = tiles[3 * tile + 1], rows = tiles[3 * tile + 2];
+  // what this thread fetches: 8 elements of one activation row and of WL weight rows per k-step
+  const int lrow = tid >> 2, lk = (tid & 3) * 8;
+  const int pos = first + min(lrow, rows - 1);  // rows beyond the tile: read again, never stored
+  const bf16_t* ap = a + (size_t)(gather ? sorted[pos] / top : pos) * a_stride;
+  const bf16_t* wp[WL];
+#pragma unroll
+  for (int i = 0; i < WL; ++i) {
+    const int r = lrow + 64 * i;  // row of the workgroup's weight tile: gate rows, then (glu) up rows
+    const int o = min(o0 + (r % MOE_BN), F - 1) + (r >= MOE_BN ? F : 0);
+    wp[i] = w + (size_t)e * N * K + (size_t)o * K;
+  }
+  moe_f32x4 acc[4][2], acc_up[4][2];
+#pragma unroll
+  for (int rt = 0; rt < 4; ++rt)
+#pragma unroll
+    for (int nt = 0; nt < 2; ++nt) acc[rt][nt] = acc_up[rt][nt] = moe_f32x4{0.f, 0.f, 0.f, 0.f};
+  moe_u32x4 ra, rw[WL];
+  auto fetch = [&](int k0) {
+    const int kk = k0 + lk, kc = min(kk, K - 8);  // loads stand under no condition; a chunk beyond the row counts as zeros
+    const uint32_t keep = kk < K ? 0xffffffffu : 0u;
+    const moe_u32x4 x = *reinterpret_cast<const moe_u32x4*>(ap + kc);
+    ra = moe_u32x4{x[0] & keep, x[1] & keep, x[2] & keep, x[3] & keep};
+#pragma unroll
+    for (int i = 0; i < WL; ++i) rw[i] = *reinterpret_cast<const moe_u32x4*>(wp[i] + kc);
+  };
+  auto stage = [&](int buf) {
+    *reinterpret_cast<moe_u32x4*>(&sa[buf][lrow][lk]) = ra;
+#pragma unroll
+    for (int i = 0; i < WL; ++i) *reinterpret_cast<moe_u32x4*>(&sw[buf][lrow + 64 * i][lk]) = rw[i];
+  };
+  fetch(0);
+  stage(0);
+  __syncthreads();
+  int buf = 0;
+  for (int k0 = 0; k0 < K; k0 += 32) {
+    const bool more = k0 + 32 < K;
+    if (more) fetch(k0 + 32);
+    moe_u32x4 av[4], wv[2], wu[2];
+#pragma unroll
+    for (int rt = 0; rt < 4; ++rt) av[rt] = *reinterpret_cast<const moe_u32x4*>(&sa[buf][16 * rt + col][8 * g]);
+#pragma unroll
+    for (int nt = 0; nt < 2; ++nt) {
+      wv[nt] = *reinterpret_cast<const moe_u32x4*>(&sw[buf][wave * 32 + 16 * nt + col][8 * g]);
+      if (GLU) wu[nt] = *reinterpret_cast<const moe_u32x4*>(&sw[buf][MOE_BN + wave * 32 + 16 * nt + col][8 * g]);
+    }
+#pragma unroll
+    for (int rt = 0; rt < 4; ++rt)
+#pragma unroll
+      for (int nt = 0; nt < 2; ++nt) {
+        acc[rt][nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(moe_as_bf16x8(wv[nt]), moe_as_bf16x8(av[rt]), acc[rt][nt], 0, 0, 0);
+        if (GLU) acc_up[rt][nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(moe_as_bf16x8(wu[nt]), moe_as_bf16x8(av[rt]), acc_up[rt][nt], 0, 0, 0);
+      }
+    if (more) stage(buf ^ 1);  // nobody reads that buffer: every wave has passed the barrier behind the step that did
+    __syncthreads();
+    buf ^= 1;
+  }
+#pragma unroll
+  for (int rt = 0; rt < 4; ++rt) {
+    if (16 * rt + col >= rows) continue;
+#pragma unroll
+    for (int nt = 0; nt < 2; ++nt)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        const int o = o0 + wave * 32 + 16 * nt + 4 * g + r;
+        if (o < F)
+          out[(size_t)(first + 16 * rt + col) * o_stride + o] = from_float<TO>(GLU ? moe_act(acc[rt][nt][r], acc_up[rt][nt][r], act) : acc[rt][nt][r]);
+      }
+  }
+}
+
 // a [rows][K]; w [E][N][K] with N = F outputs, or with glu N = 2F: gate rows then up rows; out [P][F]
 extern "C" int lev_moe_linear(const void* a, long a_stride, const void* w, void* out, long o_stride, const int* tiles, const int* meta,
                               const int* sorted, int max_tiles, int tile_rows, int top, int gather, int K, int N, int glu, int act, int dtype,
@@ -341,27 +431,35 @@ extern "C" int lev_moe_linear(const void* a, long a_stride, const void* w, void*
 #undef MOE_SPLITK
       return lev_check_launch("moe_linear (matrix cores, K split)");
     }
-    // few tiles: one column tile a wave, so that the step has four times the waves; tiles of 64 rows: four
-    const int nt = tile_rows != MOE_TM ? 4 : max_tiles <= 64 ? 1 : 2;
-    dim3 grid(max_tiles, (F + 64 * nt - 1) / (64 * nt));
-#define MOE_LAUNCH(TO, NTV, GLUV, RTV)                                                                                                            \
-  moe_linear_mfma_kernel<TO, NTV, GLUV, RTV><<<grid, 256, 0, stream>>>((const bf16_t*)a, a_stride, (const bf16_t*)w, (TO*)out, o_stride, tiles, meta, \
-                                                                       sorted, top, gather, K, N, F, act)
-#define MOE_CASE(TO, NTV)                                                                                                                        \
+    if (tile_rows != MOE_TM) {  // tiles of 64 rows: operands through LDS
+      dim3 grid_t(max_tiles, (F + MOE_BN - 1) / MOE_BN);
+#define MOE_TILE(TO)                                                                                                                             \
   do {                                                                                                                                           \
-    if (tile_rows == MOE_TM) {                                                                                                                   \
-      if (glu) MOE_LAUNCH(TO, NTV, true, 1); else MOE_LAUNCH(TO, NTV, false, 1);                                                                 \
-    } else {                                                                                                                                     \
-      if (glu) MOE_LAUNCH(TO, 4, true, 4); else MOE_LAUNCH(TO, 4, false, 4);                                                                     \
-    }                                                                                                                                            \
+    if (glu)                                                                                                                                     \
+      moe_linear_tile_kernel<TO, true><<<grid_t, 256, 0, stream>>>((const bf16_t*)a, a_stride, (const bf16_t*)w, (TO*)out, o_stride, tiles, meta,   \
+                                                                  sorted, top, gather, K, N, F, act);                                            \
+    else                                                                                                                                         \
+      moe_linear_tile_kernel<TO, false><<<grid_t, 256, 0, stream>>>((const bf16_t*)a, a_stride, (const bf16_t*)w, (TO*)out, o_stride, tiles, meta,  \
+                                                                   sorted, top, gather, K, N, F, act);                                           \
   } while (0)
-    if (out_dtype == LEV_F32) {
-      if (nt == 1) MOE_CASE(float, 1); else MOE_CASE(float, 2);
-    } else {
-      if (nt == 1) MOE_CASE(bf16_t, 1); else MOE_CASE(bf16_t, 2);
+      if (out_dtype == LEV_F32) MOE_TILE(float); else MOE_TILE(bf16_t);
+#undef MOE_TILE
+      return lev_check_launch("moe_linear (matrix cores, tiles through LDS)");
     }
+    // many tiles of 16 rows: a wave per tile and 32 outputs, both operands straight from global memory
+    const int nt = 2;
+    dim3 grid(max_tiles, (F + 64 * nt - 1) / (64 * nt));
+#define MOE_CASE(TO)                                                                                                                             \
+  do {                                                                                                                                           \
+    if (glu)                                                                                                                                     \
+      moe_linear_mfma_kernel<TO, 2, true, 1><<<grid, 256, 0, stream>>>((const bf16_t*)a, a_stride, (const bf16_t*)w, (TO*)out, o_stride, tiles, meta, \
+                                                                      sorted, top, gather, K, N, F, act);                                        \
+    else                                                                                                                                         \
+      moe_linear_mfma_kernel<TO, 2, false, 1><<<grid, 256, 0, stream>>>((const bf16_t*)a, a_stride, (const bf16_t*)w, (TO*)out, o_stride, tiles,  \
+                                                                       meta, sorted, top, gather, K, N, F, act);                                 \
+  } while (0)
+    if (out_dtype == LEV_F32) MOE_CASE(float); else MOE_CASE(bf16_t);
 #undef MOE_CASE
-#undef MOE_LAUNCH
     return lev_check_launch("moe_linear (matrix cores)");
   }
   dim3 grid(max_tiles, (F + 15) / 16);

@@ -347,13 +347,13 @@ def nakurax_config(z):
 def tativik_config(z):
     """Latent-attention layers (queries through a latent, a rotated key part of 32, a window, sinks, gates) and layers of the
     generalized delta rule, in turn, every sublayer between two norms in two groups and behind a gate; the heads, head sizes and
-    layer count of the size, a latent of two key heads' size (at most 224, so that latent and rotated part fill a key of 256).
+    layer count of the size, a latent of three key heads' size (at most 224, so that latent and rotated part fill a key of 256).
     The feed-forward has 32 experts of a quarter of the size's inner width in 8 groups of which 4 are kept, 4 experts a token:
     a token's experts hold as much as the size's dense feed-forward."""
     import math
 
     rot = 32
-    latent = {"heads": z["heads"], "dim": z["dim"], "rot_dim": rot, "vdim": z["vdim"], "kv_rank": min(224, 2 * z["dim"]), "q_rank": z["width"] // 2,
+    latent = {"heads": z["heads"], "dim": z["dim"], "rot_dim": rot, "vdim": z["vdim"], "kv_rank": min(224, 3 * z["dim"]), "q_rank": z["width"] // 2,
               "scale": 1.0 / math.sqrt(z["dim"] + rot), "rot": {"dims": rot, "base": 500000.0}, "mask": {"size": z["window"]}}
     delta = {"heads": z["width"] // z["dim"], "dim": z["dim"], "decay_rank": 64}
     mlp = {"kind": "moe", "expert": {"ff": z["ff"] // 4}, "router": {"experts": 32, "top": 4, "groups": {"count": 8, "keep": 4}}}

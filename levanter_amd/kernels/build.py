@@ -330,5 +330,5 @@ for _hd in MFMA_ATTENTION_HEAD_DIMS:
         "lev_attention_mfma": [_P, _L, _P, _L, _P, _P, _P, _P, _P, _I, _P, _I, _P, _I, _P, _P, _L, _P, _P] + [_I] * 5 + [_F, _I, _F, _P, _I, _P],
     })
 # key / value head sizes of the attention with separate sizes that are built ahead; any other pair is built at its first use
-for _hd, _vd in ((32, 16), (16, 32), (48, 32), (64, 64), (128, 64), (128, 128), (256, 256), (32, 32), (16, 16), (64, 48), (64, 32), (80, 64), (160, 128), (256, 224)):
+for _hd, _vd in ((32, 16), (16, 32), (48, 32), (64, 64), (128, 64), (128, 128), (256, 256), (32, 32), (16, 16), (64, 48), (64, 32), (80, 64), (224, 192), (256, 224)):
     attention_values_unit(_hd, _vd)

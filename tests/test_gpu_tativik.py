@@ -98,7 +98,7 @@ def test_rotation_of_halves_in_place(dtype, H, stride, offset, dims):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("R,true_R,DR,dims,H,dk", [(32, 20, 16, 4, 3, 12), (16, 16, 16, 16, 1, 8), (128, 128, 32, 32, 4, 32), (48, 41, 8, 0, 2, 16), (224, 224, 32, 32, 16, 64)])
+@pytest.mark.parametrize("R,true_R,DR,dims,H,dk", [(32, 20, 16, 4, 3, 12), (16, 16, 16, 16, 1, 8), (64, 64, 48, 32, 5, 40), (48, 41, 8, 0, 2, 16), (224, 224, 32, 32, 16, 64)])
 def test_rotation_norm_and_write_of_single_tokens_in_one_kernel_is_the_separate_kernels_bit_for_bit(dtype, R, true_R, DR, dims, H, dk):
     g = torch.Generator().manual_seed(R + DR)
     T, ps, n_pages = 7, 16, 12
@@ -354,7 +354,7 @@ def plain_attention(H, dk, dv, runs, window, scale, q, k, v, sinks):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("H,dk,dv,window,sink", [(4, 32, 24, 24, True), (8, 48, 32, 16, True), (3, 64, 48, 70, False), (6, 24, 16, 5, True), (2, 160, 128, 200, True),
+@pytest.mark.parametrize("H,dk,dv,window,sink", [(4, 32, 24, 24, True), (8, 48, 32, 16, True), (3, 64, 48, 70, False), (6, 24, 16, 5, True), (2, 256, 224, 200, True),
                                                  (34, 32, 16, 21, True), (5, 80, 64, None, True), (3, 16, 16, 1, True)])
 def test_windowed_attention_with_sinks_prompts_portions_and_single_tokens(dtype, H, dk, dv, window, sink):
     g = torch.Generator().manual_seed(H * 100 + dk)

@@ -18,9 +18,10 @@
 #define GN_MAX_PER 32
 #define GN_MAX_GROUPS 64
 
-// sum of squares of every group: each wave adds its lanes' shares group by group, the waves' sums go through LDS
+// 1 / sqrt(mean of squares + eps) of every group: each wave adds its lanes' shares group by group, the waves' sums go through LDS
 template <int PER>
-__device__ __forceinline__ void group_square_sums(const float (&v)[PER], const int (&gid)[PER], int G, float* part /*[4][G]*/, float* total /*[G]*/) {
+__device__ __forceinline__ void group_inverse_rms(const float (&v)[PER], const int (&gid)[PER], int G, float inv_n, float eps, float* part /*[4][G]*/,
+                                                  float* total /*[G]*/) {
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   for (int g = 0; g < G; ++g) {
     float s = 0.f;
@@ -31,7 +32,7 @@ __device__ __forceinline__ void group_square_sums(const float (&v)[PER], const i
     if (lane == 0) part[wave * G + g] = s;
   }
   __syncthreads();
-  if (tid < G) total[tid] = (part[tid] + part[G + tid]) + (part[2 * G + tid] + part[3 * G + tid]);
+  if (tid < G) total[tid] = 1.0f / sqrtf(((part[tid] + part[G + tid]) + (part[2 * G + tid] + part[3 * G + tid])) * inv_n + eps);
   __syncthreads();
 }
 
@@ -61,26 +62,24 @@ group_norm_step_kernel(float* __restrict__ x, const float* __restrict__ y, const
     gid[i] = e < D ? e / group_size : -1;
   }
   if (y != nullptr) {
-    group_square_sums<PER>(z, gid, G, part, total);
+    group_inverse_rms<PER>(z, gid, G, inv_n, eps, part, total);
 #pragma unroll
     for (int i = 0; i < PER; ++i) {
       const int e = tid + GN_NT * i;
       if (e < D) {
-        const float inv = 1.0f / sqrtf(total[gid[i]] * inv_n + eps);
-        xv[i] = xv[i] + mult * (z[i] * inv * pw[i]);
+        xv[i] = xv[i] + mult * (z[i] * total[gid[i]] * pw[i]);
         if (rows == nullptr) x[(size_t)row * D + e] = xv[i];
       }
     }
     __syncthreads();  // the groups' sums are read before the next use of the scratch arrays
   }
   if (h_out != nullptr) {
-    group_square_sums<PER>(xv, gid, G, part, total);
+    group_inverse_rms<PER>(xv, gid, G, inv_n, eps, part, total);
 #pragma unroll
     for (int i = 0; i < PER; ++i) {
       const int e = tid + GN_NT * i;
       if (e < D) {
-        const float inv = 1.0f / sqrtf(total[gid[i]] * inv_n + eps);
-        h_out[(size_t)r * D + e] = from_float<TO>(xv[i] * inv * wv[i]);
+        h_out[(size_t)r * D + e] = from_float<TO>(xv[i] * total[gid[i]] * wv[i]);
       }
     }
   }

@@ -41,6 +41,23 @@ head_prepare_kernel(T* __restrict__ qk, long qk_stride, int n_norm, int hd, int 
   }
 }
 
+// Heads of 512 elements and more (a latent as wide as a quarter of the model): a workgroup of 256 threads per head instead of a
+// wave, so that a head's loads are in flight together.
+template <typename T>
+__global__ void __launch_bounds__(256)
+head_prepare_wide_kernel(T* __restrict__ qk, long qk_stride, int hd, int norm_dim, float eps, const float* __restrict__ norm_w) {
+  __shared__ float red[4];
+  T* row = qk + (size_t)blockIdx.x * qk_stride + (size_t)blockIdx.y * hd;
+  float ss = 0.f;
+  for (int d = threadIdx.x; d < hd; d += 256) {
+    const float x = to_float<T>(row[d]);
+    ss = fmaf(x, x, ss);
+  }
+  ss = block_sum<256>(ss, red);
+  const float r = 1.0f / sqrtf(ss / (float)norm_dim + eps);
+  for (int d = threadIdx.x; d < hd; d += 256) row[d] = from_float<T>(to_float<T>(row[d]) * r * (norm_w ? norm_w[d] : 1.0f));
+}
+
 extern "C" int lev_head_prepare(void* qk, long qk_stride, int n_norm, int hd, int norm_dim, float eps, void* v, long v_stride, const void* v_first,
                                 long vf_stride, int n_blend, int vd, const float* lambda, const float* norm_w, int T, int dtype,
                                 hipStream_t stream) {
@@ -50,6 +67,12 @@ extern "C" int lev_head_prepare(void* qk, long qk_stride, int n_norm, int hd, in
   LEV_REQUIRE(dtype == LEV_F32 || dtype == LEV_BF16, "head_prepare: unknown dtype %d", dtype);
   LEV_REQUIRE(n_norm + n_blend <= 65535, "head_prepare: too many heads (%d)", n_norm + n_blend);
   if (T == 0 || n_norm + n_blend == 0) return 0;
+  if (n_blend == 0 && hd >= 512) {
+    dim3 wide(T, n_norm);
+    if (dtype == LEV_F32) head_prepare_wide_kernel<float><<<wide, 256, 0, stream>>>((float*)qk, qk_stride, hd, norm_dim, eps, norm_w);
+    else head_prepare_wide_kernel<bf16_t><<<wide, 256, 0, stream>>>((bf16_t*)qk, qk_stride, hd, norm_dim, eps, norm_w);
+    return lev_check_launch("head_prepare (wide heads)");
+  }
   dim3 grid(T, n_norm + n_blend);
   if (dtype == LEV_F32)
     head_prepare_kernel<float><<<grid, 64, 0, stream>>>((float*)qk, qk_stride, n_norm, hd, norm_dim, eps, (float*)v, v_stride, (const float*)v_first,

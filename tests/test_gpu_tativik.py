@@ -131,6 +131,24 @@ def test_rotation_norm_and_write_of_single_tokens_in_one_kernel_is_the_separate_
         torch.testing.assert_close(outs[0][1].cpu().double().view(T, H, qh)[:, :, dk:], want, **tol(dtype, f32=1e-3, bf16=2e-2))
 
 
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("Q,true_Q,heads", [(1024, 1024, 1), (520, 513, 2), (2048, 2000, 1)])
+def test_rms_norm_with_a_weight_of_a_wide_head(dtype, Q, true_Q, heads):
+    """A head of 512 elements and more takes a workgroup instead of a wave (the queries' latent of a wide model)."""
+    g = torch.Generator().manual_seed(Q)
+    buf = bfn(torch.randn(5, heads * Q + 16, generator=g))
+    for h in range(heads):
+        buf[:, h * Q + true_Q:(h + 1) * Q] = 0
+    w = torch.cat([1 + 0.2 * torch.randn(true_Q, generator=g), torch.zeros(Q - true_Q)])
+    b = dev(buf, dtype)
+    K().head_prepare(b, heads, Q, 1e-5, norm_dim=true_Q, norm_weight=w.to(DEV))
+    got = b.cpu().double()
+    for h in range(heads):
+        torch.testing.assert_close(got[:, h * Q:h * Q + true_Q], P.rms_norm(buf[:, h * Q:h * Q + true_Q], w[:true_Q].double(), 1e-5), **tol(dtype))
+        assert not got[:, h * Q + true_Q:(h + 1) * Q].any()
+    assert torch.equal(got[:, heads * Q:], buf[:, heads * Q:])
+
+
 def delta_inputs(T, H, d, g, dtype):
     C = H * d
     stride = 5 * C + 8

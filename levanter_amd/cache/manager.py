@@ -106,8 +106,9 @@ class PagedGroup:
             return 0
         first_needed = self.requirement.first_needed(length)
         first_block = first_needed // self.page_size
+        kept_blocks = self.kept_blocks()  # the blocks of the first positions that stay readable are never given back
         n = 0
-        for b in range(int(self.first_live_block[slot]), first_block):
+        for b in range(max(int(self.first_live_block[slot]), kept_blocks), first_block):
             page = int(self.block_tables[slot, b])
             if page != NO_PAGE:
                 self.pool.free(page)
@@ -115,6 +116,10 @@ class PagedGroup:
                 n += 1
         self.first_live_block[slot] = max(int(self.first_live_block[slot]), first_block)
         return n
+
+    def kept_blocks(self) -> int:
+        """Blocks at a request's start that hold positions every later query may read."""
+        return (self.requirement.keep_first + self.page_size - 1) // self.page_size
 
     def release_all(self, slot: int) -> None:
         row = self.block_tables[slot]
@@ -301,7 +306,8 @@ class CacheManager:
                 hi = (h.length + self.page_size - 1) // self.page_size
                 row = g.block_tables[slot]
                 assert (row[lo:hi] != NO_PAGE).all(), f"slot {slot}: a live block has no page"
-                assert (row[:lo] == NO_PAGE).all(), f"slot {slot}: a block behind the window still has a page"
+                assert (row[min(g.kept_blocks(), lo):lo] == NO_PAGE).all(), f"slot {slot}: a block behind the window still has a page"
+                assert (row[:min(g.kept_blocks(), lo, hi)] != NO_PAGE).all(), f"slot {slot}: a block of the kept first positions has no page"
         assert len(set(self._free_slots)) == len(self._free_slots)
         assert set(self._free_slots).isdisjoint(self.live.keys())
         assert len(self._free_slots) + len(self.live) == self.max_seqs

@@ -15,6 +15,7 @@ class PagedKv:
     window: Optional[int] = None  # None: all keys. w: a query at position p reads keys p-w+1 .. p
     value_dim: Optional[int] = None  # size of a value head where it differs from a key head's (None: head_dim)
     chunk: Optional[int] = None  # c: a query at position p reads only keys of its own chunk, (p // c) * c .. p
+    keep_first: int = 0  # the first so many positions of a request stay readable whatever window and chunk say
 
     @property
     def v_dim(self) -> int:
@@ -24,7 +25,7 @@ class PagedKv:
     def reach(self) -> Optional[int]:
         """The most keys any query reads (None: all keys so far)."""
         both = [n for n in (self.window, self.chunk) if n is not None]
-        return min(both) if both else None
+        return min(both) + self.keep_first if both else None
 
     def first_needed(self, length: int) -> int:
         """The first position that a query at position ``length`` or later can still read."""

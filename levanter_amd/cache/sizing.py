@@ -26,7 +26,7 @@ def group_page_bytes(req: PagedKv, n_units: int, page_size: int, itemsize: int) 
 def window_group_pages(req: PagedKv, page_size: int, max_seqs: int, max_pages_per_seq: int, longest_portion: int) -> int:
     """The most pages a windowed group can hold at once: per live request the blocks that the window and one step's
     portion touch (one more for a window that starts inside a block), never more than a request's table has."""
-    per_seq = (req.reach + longest_portion + page_size - 1) // page_size + 1
+    per_seq = (req.reach + longest_portion + page_size - 1) // page_size + 1 + (1 if req.keep_first else 0)  # kept first positions end inside a block
     return max_seqs * min(per_seq, max_pages_per_seq)
 
 

@@ -13,6 +13,7 @@
 //   score(t, key) = cap(scale * q . k) - slope[h] * (position(t) - position(key)),  cap(s) = softcap * tanh(s / softcap)
 //   a query at position p sees keys max(0, p - window + 1) .. p (window 0: all) and, with chunk > 0, only keys of its own
 //   chunk of positions, (p / chunk) * chunk .. p (chunks are counted from position 0). A key whose block has no page is masked.
+//   keep > 0: the first `keep` positions of the sequence are seen by every later query as well, at their true distances.
 //   sinks (float32 [H] or null): the softmax's denominator of head h also holds exp(sinks[h]), once per query: a score without
 //   a key and without a value, neither scaled nor capped.
 // One wave per (query token, head); keys are visited 64 at a time.
@@ -26,7 +27,7 @@ __global__ void __launch_bounds__(64)
 attention_values_kernel(const T* __restrict__ q, long q_stride, float* __restrict__ out, const T* __restrict__ k_pages,
                         const T* __restrict__ v_pages, const int* __restrict__ positions, const int* __restrict__ token_seq,
                         const int* __restrict__ block_tables, int bt_stride, int H, int KVH, int HD, int VD, int NV, int PS, float scale,
-                        int window, int chunk, float softcap, const float* __restrict__ slopes, const float* __restrict__ sinks) {
+                        int window, int chunk, int keep, float softcap, const float* __restrict__ slopes, const float* __restrict__ sinks) {
   __shared__ float qs[AV_MAX_HD];
   __shared__ float ps[64];
   __shared__ int pg[64];
@@ -48,9 +49,11 @@ attention_values_kernel(const T* __restrict__ q, long q_stride, float* __restric
   float m = -INFINITY, l = 0.f;
   __syncthreads();
   const size_t k_head = (size_t)HD * PS, v_head = (size_t)VD * PS;
-  for (int c0 = (first / 64) * 64; c0 <= pos; c0 += 64) {
+  const int first_block = first / 64, n_kept = lev_kept_blocks(first, keep), n_blocks = n_kept + pos / 64 - first_block + 1;
+  for (int bi = 0; bi < n_blocks; ++bi) {
+    const int c0 = lev_block_key(bi, n_kept, first_block);
     const int kp = c0 + lane;
-    bool live = kp >= first && kp <= pos;
+    bool live = lev_key_visible(kp, pos, first, keep);
     float s = -INFINITY;
     int page = -1;
     if (live) page = bt[kp / PS];
@@ -103,7 +106,7 @@ attention_values_kernel(const T* __restrict__ q, long q_stride, float* __restric
 
 extern "C" int lev_attention_values(const void* q, long q_stride, float* out, const void* k_pages, const void* v_pages,
                                     const int* positions, const int* token_seq, const int* block_tables, int bt_stride, int T, int H,
-                                    int KVH, int HD, int VD, int NV, int PS, float scale, int window, int chunk, float softcap,
+                                    int KVH, int HD, int VD, int NV, int PS, float scale, int window, int chunk, int keep, float softcap,
                                     const float* slopes, const float* sinks, int dtype, hipStream_t stream) {
   LEV_REQUIRE(T >= 0 && H > 0 && KVH > 0 && H % KVH == 0, "attention: bad head counts heads=%d kv_heads=%d", H, KVH);
   LEV_REQUIRE(HD > 0 && HD % 8 == 0 && HD <= AV_MAX_HD, "attention: head_dim=%d must be a multiple of 8 and at most %d", HD, AV_MAX_HD);
@@ -111,7 +114,7 @@ extern "C" int lev_attention_values(const void* q, long q_stride, float* out, co
   LEV_REQUIRE(VD <= 64 * AV_MAX_ACC, "attention: a value head of %d exceeds the %d outputs a wave may have", VD, 64 * AV_MAX_ACC);
   LEV_REQUIRE(PS > 0 && PS % 16 == 0, "attention: page_size=%d must be a multiple of 16", PS);
   LEV_REQUIRE(H <= 65535, "attention: too many heads (%d)", H);
-  LEV_REQUIRE(window >= 0 && chunk >= 0 && softcap >= 0.f, "attention: window=%d, chunk=%d and soft cap %g must not be negative", window, chunk, (double)softcap);
+  LEV_REQUIRE(window >= 0 && chunk >= 0 && keep >= 0 && softcap >= 0.f, "attention: window=%d, chunk=%d, kept positions %d and soft cap %g must not be negative", window, chunk, keep, (double)softcap);
   LEV_REQUIRE(dtype == LEV_F32 || dtype == LEV_BF16, "attention: unknown dtype %d", dtype);
   if (T == 0) return 0;
   const int per_wave = NV == 1 ? 1 : (64 * AV_MAX_ACC) / VD;
@@ -119,10 +122,10 @@ extern "C" int lev_attention_values(const void* q, long q_stride, float* out, co
   if (dtype == LEV_F32)
     attention_values_kernel<float><<<grid, 64, 0, stream>>>((const float*)q, q_stride, out, (const float*)k_pages, (const float*)v_pages,
                                                            positions, token_seq, block_tables, bt_stride, H, KVH, HD, VD, NV, PS, scale,
-                                                           window, chunk, softcap, slopes, sinks);
+                                                           window, chunk, keep, softcap, slopes, sinks);
   else
     attention_values_kernel<bf16_t><<<grid, 64, 0, stream>>>((const bf16_t*)q, q_stride, out, (const bf16_t*)k_pages,
                                                             (const bf16_t*)v_pages, positions, token_seq, block_tables, bt_stride, H, KVH,
-                                                            HD, VD, NV, PS, scale, window, chunk, softcap, slopes, sinks);
+                                                            HD, VD, NV, PS, scale, window, chunk, keep, softcap, slopes, sinks);
   return lev_check_launch("attention_values");
 }

@@ -64,7 +64,7 @@ __global__ void __launch_bounds__(64)
 attention_values_mfma_kernel(const bf16_t* __restrict__ q, long q_stride, float* __restrict__ out, const bf16_t* __restrict__ k_pages,
                              const bf16_t* __restrict__ v_pages, const int* __restrict__ positions, const int* __restrict__ token_seq,
                              const int* __restrict__ block_tables, int bt_stride, const int* __restrict__ work, int H, int KVH, int NV,
-                             int PS, float scale, int window, int chunk, float softcap, const float* __restrict__ slopes, int splits,
+                             int PS, float scale, int window, int chunk, int keep, float softcap, const float* __restrict__ slopes, int splits,
                              float* __restrict__ part_o, float* __restrict__ part_ml, const float* __restrict__ sinks) {
   const int lane = threadIdx.x, col = lane & 15, g = lane >> 4;
   const int group = H / KVH;
@@ -117,13 +117,16 @@ attention_values_mfma_kernel(const bf16_t* __restrict__ q, long q_stride, float*
   const size_t k_head = (size_t)HD * PS, v_head = (size_t)VD * PS;
 
   // a single token's keys may be split over `splits` waves (blockIdx.x % splits): each takes a run of whole blocks
-  int key_first = (lo_min / 64) * 64, key_last = p_max;
+  // the blocks of 64 keys: those of the kept first positions that lie before the window's first block, then the window's
+  const int first_block = lo_min / 64, n_kept = lev_kept_blocks(lo_min, keep);
+  int block_first = 0, block_last = n_kept + p_max / 64 - first_block;
   if (SINGLE && splits > 1) {
-    const int n_blocks = p_max / 64 - lo_min / 64 + 1, per = (n_blocks + splits - 1) / splits, z = blockIdx.x % splits;
-    key_first += z * per * 64;
-    key_last = min(p_max, key_first + per * 64 - 1);
+    const int per = (block_last + splits) / splits, z = blockIdx.x % splits;
+    block_first = z * per;
+    block_last = min(block_last, block_first + per - 1);
   }
-  for (int key0 = key_first; key0 <= key_last; key0 += 64) {
+  for (int bi = block_first; bi <= block_last; ++bi) {
+    const int key0 = lev_block_key(bi, n_kept, first_block);
     // pages of this lane's two groups of 8 keys (32u + 8g .. +7): for the mask and for the values
     int pgv[2];
 #pragma unroll
@@ -160,7 +163,7 @@ attention_values_mfma_kernel(const bf16_t* __restrict__ q, long q_stride, float*
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
           const int kp = key0 + 32 * u + 8 * g + 4 * hh + r;
-          const bool ok = valid && kp <= pos && kp >= lo && pgv[u] >= 0;
+          const bool ok = valid && lev_key_visible(kp, pos, lo, keep) && pgv[u] >= 0;
           float s = st[u][hh][r] * scale;
           if (softcap > 0.f) s = softcap * fast_tanh(s * __builtin_amdgcn_rcpf(softcap));
           s = (s - slope * (float)(pos - kp)) * LOG2E;
@@ -254,7 +257,7 @@ __global__ void __launch_bounds__(PF_THREADS)
 attention_values_mfma_runs_kernel(const bf16_t* __restrict__ q, long q_stride, float* __restrict__ out, const bf16_t* __restrict__ k_pages,
                                   const bf16_t* __restrict__ v_pages, const int* __restrict__ positions, const int* __restrict__ token_seq,
                                   const int* __restrict__ block_tables, int bt_stride, const int* __restrict__ tiles, int H, int KVH, int NV,
-                                  int PS, float scale, int window, int chunk, float softcap, const float* __restrict__ slopes,
+                                  int PS, float scale, int window, int chunk, int keep, float softcap, const float* __restrict__ slopes,
                                   const float* __restrict__ sinks) {
   extern __shared__ __attribute__((aligned(16))) unsigned char av_smem[];
   bf16_t* ks = reinterpret_cast<bf16_t*>(av_smem);  // [HD/8][64][8]
@@ -284,9 +287,17 @@ attention_values_mfma_runs_kernel(const bf16_t* __restrict__ q, long q_stride, f
   const int sh = (PS & (PS - 1)) == 0 ? __builtin_ctz(PS) : -1;
   const int pg0 = sh >= 0 ? key_begin >> sh : key_begin / PS;
   const int n_pg = (sh >= 0 ? p_max_wg >> sh : p_max_wg / PS) - pg0 + 1;
-  for (int i = tid; i < min(n_pg, RUN_PAGES); i += PF_THREADS) pages_s[i] = bt[pg0 + i];  // the host sends longer ranges elsewhere
+  // with kept first positions the tile also reads the n_kept blocks of 64 keys that hold them and lie before key_begin: their
+  // page ids stand at the table's start, those of the range from key_begin on behind them
+  const int first_block = lo_wg / 64, n_kept = lev_kept_blocks(lo_wg, keep), n_blocks = n_kept + p_max_wg / 64 - first_block + 1;
+  const int n_kpg = n_kept > 0 ? (sh >= 0 ? (n_kept * 64 - 1) >> sh : (n_kept * 64 - 1) / PS) + 1 : 0;
+  for (int i = tid; i < min(n_kpg, RUN_PAGES); i += PF_THREADS) pages_s[i] = bt[i];
+  for (int i = tid; i < min(n_pg, RUN_PAGES - n_kpg); i += PF_THREADS) pages_s[n_kpg + i] = bt[pg0 + i];  // the host sends longer ranges elsewhere
   auto block_of = [&](int kp) { return sh >= 0 ? kp >> sh : kp / PS; };
-  auto page_of = [&](int kp) { return pages_s[block_of(kp) - pg0]; };  // kp within the tile's range
+  auto page_of = [&](int kp) {  // kp within the tile's range or among the kept blocks
+    const int b = block_of(kp);
+    return pages_s[b >= pg0 ? n_kpg + b - pg0 : b];
+  };
 
   u32x4 qf[NKS];
 #pragma unroll
@@ -344,22 +355,23 @@ attention_values_mfma_runs_kernel(const bf16_t* __restrict__ q, long q_stride, f
     }
   };
 
-  fetch(key_begin, kst_a, vst_a);
-  if (key_begin + 64 <= p_max_wg) fetch(key_begin + 64, kst_b, vst_b);
-  for (int key0 = key_begin, it = 0; key0 <= p_max_wg; key0 += 64, ++it) {
+  fetch(lev_block_key(0, n_kept, first_block), kst_a, vst_a);
+  if (n_blocks > 1) fetch(lev_block_key(1, n_kept, first_block), kst_b, vst_b);
+  for (int it = 0; it < n_blocks; ++it) {
+    const int key0 = lev_block_key(it, n_kept, first_block);
     lds_barrier();  // the block before has been read by every wave (a barrier for LDS only: the loads on their way stay there)
     // the register sets take turns: this block's goes to LDS and is asked for again two blocks ahead (conditions uniform
     // over the workgroup)
     if (it & 1) {
       stage(kst_b, vst_b);
       lds_barrier();
-      if (key0 + 128 <= p_max_wg) fetch(key0 + 128, kst_b, vst_b);
+      if (it + 2 < n_blocks) fetch(lev_block_key(it + 2, n_kept, first_block), kst_b, vst_b);
     } else {
       stage(kst_a, vst_a);
       lds_barrier();
-      if (key0 + 128 <= p_max_wg) fetch(key0 + 128, kst_a, vst_a);
+      if (it + 2 < n_blocks) fetch(lev_block_key(it + 2, n_kept, first_block), kst_a, vst_a);
     }
-    if (!active || key0 > p_max || key0 + 63 < lo_min) continue;  // none of this wave's rows sees a key of this block
+    if (!active || key0 > p_max || (key0 + 63 < lo_min && key0 >= keep)) continue;  // none of this wave's rows sees a key of this block
     int pgv[2];
 #pragma unroll
     for (int u = 0; u < 2; ++u) {
@@ -390,7 +402,7 @@ attention_values_mfma_runs_kernel(const bf16_t* __restrict__ q, long q_stride, f
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
           const int kp = key0 + 32 * u + 8 * g + 4 * hh + r;
-          const bool ok = valid && kp <= pos && kp >= lo && pgv[u] >= 0;
+          const bool ok = valid && lev_key_visible(kp, pos, lo, keep) && pgv[u] >= 0;
           float sc = st[u][hh][r] * scale;
           if (softcap > 0.f) sc = softcap * fast_tanh(sc * __builtin_amdgcn_rcpf(softcap));
           sc = (sc - slope * (float)(pos - kp)) * LOG2E;
@@ -490,13 +502,13 @@ extern "C" long lev_attention_values_mfma_workspace(int n_singles, int splits, i
 extern "C" int lev_attention_values_mfma(const void* q, long q_stride, float* out, const void* k_pages, const void* v_pages,
                                          const int* positions, const int* token_seq, const int* block_tables, int bt_stride,
                                          const int* tiles, int n_tiles, const int* singles, int n_singles, int H, int KVH, int HD_,
-                                         int VD_, int NV, int PS, float scale, int window, int chunk, float softcap, const float* slopes,
+                                         int VD_, int NV, int PS, float scale, int window, int chunk, int keep, float softcap, const float* slopes,
                                          const float* sinks, int splits, float* workspace, int max_keys, hipStream_t stream) {
   LEV_REQUIRE(HD_ == HD && VD_ == VD, "attention: this library was built for head sizes %d / %d, not %d / %d", HD, VD, HD_, VD_);
   LEV_REQUIRE(H > 0 && KVH > 0 && H % KVH == 0, "attention: bad head counts heads=%d kv_heads=%d", H, KVH);
   LEV_REQUIRE(NV == 1 || NV == KVH, "attention: %d value heads per query head (1 or kv_heads=%d)", NV, KVH);
   LEV_REQUIRE(PS > 0 && PS % 16 == 0, "attention: page_size=%d must be a multiple of 16", PS);
-  LEV_REQUIRE(window >= 0 && chunk >= 0 && softcap >= 0.f, "attention: window=%d, chunk=%d and soft cap %g must not be negative", window, chunk, (double)softcap);
+  LEV_REQUIRE(window >= 0 && chunk >= 0 && keep >= 0 && softcap >= 0.f, "attention: window=%d, chunk=%d, kept positions %d and soft cap %g must not be negative", window, chunk, keep, (double)softcap);
   LEV_REQUIRE(splits >= 1 && splits <= MERGE_MAX_SPLITS && (splits == 1 || workspace), "attention: %d splits (at most %d) need scratch memory", splits,
               MERGE_MAX_SPLITS);
   LEV_REQUIRE(n_tiles >= 0 && n_singles >= 0 && (n_tiles == 0 || tiles) && (n_singles == 0 || singles), "attention: bad work lists");
@@ -511,15 +523,15 @@ extern "C" int lev_attention_values_mfma(const void* q, long q_stride, float* ou
     // the page ids of a tile's key range (the window, or all keys so far, and the tile itself) must fit their LDS table
     long reach = window > 0 && window < max_keys ? window : max_keys;
     if (chunk > 0 && chunk < reach) reach = chunk;
-    reach += PF_ROWS + 64;
+    reach += PF_ROWS + 64 + (keep > 0 ? keep + 64 + PS : 0);
     if (lds + RUN_PAGES * sizeof(int) <= 64 * 1024 && reach / PS + 2 <= RUN_PAGES)
       attention_values_mfma_runs_kernel<<<grid, PF_THREADS, lds, stream>>>((const bf16_t*)q, q_stride, out, (const bf16_t*)k_pages,
                                                                          (const bf16_t*)v_pages, positions, token_seq, block_tables,
-                                                                         bt_stride, tiles, H, KVH, NV, PS, scale, window, chunk, softcap, slopes, sinks);
+                                                                         bt_stride, tiles, H, KVH, NV, PS, scale, window, chunk, keep, softcap, slopes, sinks);
     else  // the largest head sizes, the longest ranges: every wave by itself, operands straight from the pages
       attention_values_mfma_kernel<false><<<dim3(n_tiles * SUB_TILES, H, chunks), 64, 0, stream>>>(
           (const bf16_t*)q, q_stride, out, (const bf16_t*)k_pages, (const bf16_t*)v_pages, positions, token_seq, block_tables, bt_stride,
-          tiles, H, KVH, NV, PS, scale, window, chunk, softcap, slopes, 1, nullptr, nullptr, sinks);
+          tiles, H, KVH, NV, PS, scale, window, chunk, keep, softcap, slopes, 1, nullptr, nullptr, sinks);
     if (lev_check_launch("attention_values_mfma (runs)")) return -1;
   }
   if (n_singles > 0) {
@@ -529,7 +541,7 @@ extern "C" int lev_attention_values_mfma(const void* q, long q_stride, float* ou
     float* part_ml = splits > 1 ? workspace + (size_t)n_singles * splits * H * NV * VD : nullptr;
     attention_values_mfma_kernel<true><<<grid, 64, 0, stream>>>((const bf16_t*)q, q_stride, out, (const bf16_t*)k_pages,
                                                                (const bf16_t*)v_pages, positions, token_seq, block_tables, bt_stride,
-                                                               singles, H, KVH, NV, PS, scale, window, chunk, softcap, slopes, splits, part_o,
+                                                               singles, H, KVH, NV, PS, scale, window, chunk, keep, softcap, slopes, splits, part_o,
                                                                part_ml, sinks);
     if (lev_check_launch("attention_values_mfma (single tokens)")) return -1;
     if (splits > 1) {

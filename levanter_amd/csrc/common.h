@@ -104,6 +104,18 @@ __host__ __device__ __forceinline__ int lev_first_visible(int pos, int window, i
   return lo;
 }
 
+// With `keep` > 0 the first `keep` positions of a sequence stay in sight of every later query, whatever the window or chunk
+// (lo is what lev_first_visible gives for the query at pos).
+__host__ __device__ __forceinline__ bool lev_key_visible(int kp, int pos, int lo, int keep) { return kp <= pos && (kp >= lo || kp < keep); }
+// The blocks of 64 keys that a set of queries reads are then two stretches: the blocks that hold kept positions and lie wholly
+// before the block of the earliest window start lo_min (their number comes back), and the blocks from that one on.
+__host__ __device__ __forceinline__ int lev_kept_blocks(int lo_min, int keep) {
+  const int kb = (keep + 63) / 64, wb = lo_min / 64;
+  return kb < wb ? kb : wb;
+}
+// the first key of the i-th block of such a list (first_block: the block of lo_min)
+__host__ __device__ __forceinline__ int lev_block_key(int i, int n_kept, int first_block) { return (i < n_kept ? i : first_block + (i - n_kept)) * 64; }
+
 // ---- activation functions, in 32-bit --------------------------------------------------------
 // x / (1 + 2^t) with the hardware's exp2 and reciprocal (about 1 ulp each): a handful of instructions where expf and
 // an IEEE division take thirty. 2^t = inf gives u * 0, the right limit.

@@ -47,6 +47,54 @@ extern "C" int lev_embed(const int* tokens, const int* positions, const void* ta
 }
 
 // ------------------------------------------------------------------------------------------
+// An embedding of the pair (token before, token), added to the stream: x[t, :] += float(table[row_t, :]) with
+//     row_t = (previous * mul_prev + token * mul_cur) mod buckets,   or row `buckets` (the table's last) at position 0.
+// The token before is the step's own token t - 1 where that one belongs to the same request and stands one position earlier,
+// else what the request's slot holds in `last_token` (the last token of the step before). A second kernel, launched behind the
+// first, stores each run's last token there. Tokens of nobody (slot < 0) read row `buckets` and store nothing.
+template <typename T>
+__global__ void __launch_bounds__(256)
+pair_embed_add_kernel(const int* __restrict__ tokens, const int* __restrict__ positions, const int* __restrict__ token_slots,
+                      const int* __restrict__ last_token, const T* __restrict__ table, float* __restrict__ x, int D, int buckets, long mul_prev,
+                      long mul_cur) {
+  const int t = blockIdx.x;
+  const int slot = token_slots[t], pos = positions[t];
+  int row = buckets;
+  if (slot >= 0 && pos > 0) {
+    const bool inside = t > 0 && token_slots[t - 1] == slot && positions[t - 1] == pos - 1;
+    const long prev = inside ? tokens[t - 1] : last_token[slot];
+    row = (int)((prev * mul_prev + (long)tokens[t] * mul_cur) % (long)buckets);
+    if (row < 0) row += buckets;
+  }
+  const T* r = table + (size_t)row * D;
+  float* o = x + (size_t)t * D;
+  for (int d = threadIdx.x; d < D; d += 256) o[d] += to_float<T>(r[d]);
+}
+
+__global__ void __launch_bounds__(256)
+last_token_store_kernel(const int* __restrict__ tokens, const int* __restrict__ token_slots, int* __restrict__ last_token, int Tn) {
+  const int t = blockIdx.x * 256 + threadIdx.x;
+  if (t >= Tn) return;
+  const int slot = token_slots[t];
+  if (slot >= 0 && (t + 1 >= Tn || token_slots[t + 1] != slot)) last_token[slot] = tokens[t];
+}
+
+extern "C" int lev_pair_embed_add(const int* tokens, const int* positions, const int* token_slots, int* last_token, const void* table, float* x,
+                                  int T, int D, int buckets, long mul_prev, long mul_cur, int dtype, hipStream_t stream) {
+  LEV_REQUIRE(T >= 0 && D > 0 && buckets > 0, "pair embedding: bad sizes T=%d D=%d buckets=%d", T, D, buckets);
+  LEV_REQUIRE(tokens && positions && token_slots && last_token && table && x, "pair embedding: a tensor is missing");
+  LEV_REQUIRE(dtype == LEV_F32 || dtype == LEV_BF16, "pair embedding: unknown dtype %d", dtype);
+  if (T == 0) return 0;
+  if (dtype == LEV_F32)
+    pair_embed_add_kernel<float><<<T, 256, 0, stream>>>(tokens, positions, token_slots, last_token, (const float*)table, x, D, buckets, mul_prev, mul_cur);
+  else
+    pair_embed_add_kernel<bf16_t><<<T, 256, 0, stream>>>(tokens, positions, token_slots, last_token, (const bf16_t*)table, x, D, buckets, mul_prev, mul_cur);
+  if (lev_check_launch("pair_embed_add")) return -1;
+  last_token_store_kernel<<<(T + 255) / 256, 256, 0, stream>>>(tokens, token_slots, last_token, T);
+  return lev_check_launch("last_token_store");
+}
+
+// ------------------------------------------------------------------------------------------
 // One block per output row. Statistics in 32-bit, two passes (mean, then the centred squares).
 // rows != null: output row r is the norm of input row rows[r] (the wanted rows before the head).
 // Rows of up to NT * 4 * NV floats are read once, as float4, into registers: every load of the row is in

@@ -8,7 +8,8 @@
 //                                                              element by the sigmoid of gate (float32 or compute dtype, row stride
 //                                                              gate_stride; null: not gated), normalised and added to the residual
 //   read:   h = gn(x, w)                                       for the next sublayer, into h_out (compute dtype or float32; may be x
-//                                                              itself when there is no write)
+//                                                              itself when there is no write); w == null: h = x as it is, only
+//                                                              rounded to h_out's type (a sublayer that reads the stream itself)
 //   rows != null: only these rows (output row r is row rows[r]); x is not stored then: a selection may name a row twice, and
 //                 the rows left out stay behind anyway.
 // All statistics and sums are 32-bit. One workgroup of 256 threads per row; the row lives in registers (D <= 256 * GN_MAX_PER).
@@ -55,7 +56,7 @@ group_norm_step_kernel(float* __restrict__ x, const float* __restrict__ y, const
     xv[i] = x[(size_t)row * D + ec];
     z[i] = y != nullptr ? y[(size_t)row * D + ec] : 0.f;
     pw[i] = y != nullptr ? post_w[ec] : 0.f;
-    wv[i] = h_out != nullptr ? w[ec] : 0.f;
+    wv[i] = (h_out != nullptr && w != nullptr) ? w[ec] : 0.f;
     const float gt = gate != nullptr ? to_float<TG>(gate[(size_t)row * gate_stride + ec]) : 0.f;
     if (gate != nullptr) z[i] = z[i] / (1.0f + expf(-gt));
     if (e >= D) xv[i] = 0.f, z[i] = 0.f;
@@ -73,7 +74,13 @@ group_norm_step_kernel(float* __restrict__ x, const float* __restrict__ y, const
     }
     __syncthreads();  // the groups' sums are read before the next use of the scratch arrays
   }
-  if (h_out != nullptr) {
+  if (h_out != nullptr && w == nullptr) {
+#pragma unroll
+    for (int i = 0; i < PER; ++i) {
+      const int e = tid + GN_NT * i;
+      if (e < D) h_out[(size_t)r * D + e] = from_float<TO>(xv[i]);
+    }
+  } else if (h_out != nullptr) {
     group_inverse_rms<PER>(xv, gid, G, inv_n, eps, part, total);
 #pragma unroll
     for (int i = 0; i < PER; ++i) {
@@ -104,7 +111,7 @@ extern "C" int lev_group_norm_step(float* x, const float* y, const void* gate, l
                                    hipStream_t stream) {
   LEV_REQUIRE(n >= 0 && D > 0 && D <= GN_NT * GN_MAX_PER, "group norm: a row of %d numbers (at most %d)", D, GN_NT * GN_MAX_PER);
   LEV_REQUIRE(G > 0 && G <= GN_MAX_GROUPS && D % G == 0, "group norm: %d numbers do not split into %d equal groups (at most %d)", D, G, GN_MAX_GROUPS);
-  LEV_REQUIRE(x != nullptr && (y == nullptr || post_w != nullptr) && (h_out == nullptr || w != nullptr), "group norm: a tensor is missing");
+  LEV_REQUIRE(x != nullptr && (y == nullptr || post_w != nullptr), "group norm: a tensor is missing");
   LEV_REQUIRE(y != nullptr || h_out != nullptr, "group norm: nothing to do");
   LEV_REQUIRE(gate == nullptr || (y != nullptr && gate_stride >= D), "group norm: a gate needs a result to gate and rows of at least %d", D);
   LEV_REQUIRE((gate_dtype == LEV_F32 || gate_dtype == LEV_BF16) && (out_dtype == LEV_F32 || out_dtype == LEV_BF16), "group norm: unknown dtype");

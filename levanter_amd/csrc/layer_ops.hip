@@ -88,14 +88,17 @@ extern "C" int lev_head_prepare(void* qk, long qk_stride, int n_norm, int hd, in
 // item); items are the H query heads (normalised in place), the G key heads (normalised, written to the key pages
 // [page][G][hd/8][PS][8]) and the G value heads (blended, written to the value pages [page][G][vd][PS]). dest[t] =
 // page * PS + offset, negative for a token that is written nowhere. norm_dim: the divisor of the mean of squares (the head's
-// true size); 0: queries and keys stay as they are.
+// true size); 0: queries and keys stay as they are. q_norm_w / k_norm_w (float32 [hd], or null): the normalised query / key
+// heads are multiplied by it (an RMS norm with a weight, one for all heads of a kind). magnitude: cosine and sine of the
+// rotation are both multiplied by it.
 template <typename T>
 __global__ void __launch_bounds__(64)
 head_prepare_write_kernel(T* __restrict__ q, long q_stride, int H, const T* __restrict__ k, long k_stride, const T* __restrict__ v,
                           long v_stride, const T* __restrict__ v_first, long vf_stride, const float* __restrict__ lambda, int G, int hd,
                           int vd, float eps, int norm_dim, T* __restrict__ k_pages, T* __restrict__ v_pages,
                           const int* __restrict__ dest, int PS, const float* __restrict__ freqs, int n_pairs,
-                          const int* __restrict__ positions) {
+                          const int* __restrict__ positions, const float* __restrict__ q_norm_w, const float* __restrict__ k_norm_w,
+                          float magnitude) {
   const int t = blockIdx.x, item = blockIdx.y, lane = threadIdx.x;
   if (item < H + G) {
     const bool is_q = item < H;
@@ -115,6 +118,7 @@ head_prepare_write_kernel(T* __restrict__ q, long q_stride, int H, const T* __re
     const int dst = is_q ? 0 : dest[t];
     if (dst < 0) return;
     const float pos = freqs ? (float)positions[t] : 0.f;
+    const float* norm_w = is_q ? q_norm_w : k_norm_w;
     T* qrow = q + (size_t)t * q_stride + (size_t)item * hd;
     T* kd = is_q ? nullptr : k_pages + ((size_t)(dst / PS) * G + (item - H)) * (size_t)hd * PS;
     const int off = dst % PS;
@@ -124,9 +128,11 @@ head_prepare_write_kernel(T* __restrict__ q, long q_stride, int H, const T* __re
       if (normalise || i < n_pairs) {
         float a = to_float<T>(e0), b = to_float<T>(e1);
         if (normalise) a *= r, b *= r;
+        if (normalise && norm_w) a *= norm_w[2 * i], b *= norm_w[2 * i + 1];
         if (i < n_pairs) {
           float sn, cs;
           sincosf(pos * freqs[i], &sn, &cs);
+          sn *= magnitude, cs *= magnitude;
           const float ra = a * cs - b * sn, rb = b * cs + a * sn;
           a = ra, b = rb;
         }
@@ -161,7 +167,8 @@ head_prepare_write_kernel(T* __restrict__ q, long q_stride, int H, const T* __re
 extern "C" int lev_head_prepare_write(void* q, long q_stride, int H, const void* k, long k_stride, const void* v, long v_stride,
                                       const void* v_first, long vf_stride, const float* lambda, int G, int hd, int vd, float eps,
                                       int norm_dim, void* k_pages, void* v_pages, const int* dest, int PS, const float* freqs, int n_pairs,
-                                      const int* positions, int T, int dtype, hipStream_t stream) {
+                                      const int* positions, const float* q_norm_w, const float* k_norm_w, float magnitude, int T, int dtype,
+                                      hipStream_t stream) {
   LEV_REQUIRE(n_pairs >= 0 && 2 * n_pairs <= hd && (n_pairs == 0 || (freqs && positions)), "head_prepare_write: %d rotated pairs need frequencies, positions and a head of at least twice their number", n_pairs);
   LEV_REQUIRE(T >= 0 && H > 0 && G > 0 && hd > 0 && hd % 8 == 0 && vd > 0, "head_prepare_write: bad sizes T=%d heads=%d/%d sizes=%d/%d", T, H, G, hd, vd);
   LEV_REQUIRE(q && k && v && k_pages && v_pages && dest, "head_prepare_write: a tensor is missing");
@@ -175,11 +182,13 @@ extern "C" int lev_head_prepare_write(void* q, long q_stride, int H, const void*
   if (dtype == LEV_F32)
     head_prepare_write_kernel<float><<<grid, 64, 0, stream>>>((float*)q, q_stride, H, (const float*)k, k_stride, (const float*)v, v_stride,
                                                              (const float*)v_first, vf_stride, lambda, G, hd, vd, eps, norm_dim,
-                                                             (float*)k_pages, (float*)v_pages, dest, PS, freqs, n_pairs, positions);
+                                                             (float*)k_pages, (float*)v_pages, dest, PS, freqs, n_pairs, positions, q_norm_w, k_norm_w,
+                                                             magnitude);
   else
     head_prepare_write_kernel<bf16_t><<<grid, 64, 0, stream>>>((bf16_t*)q, q_stride, H, (const bf16_t*)k, k_stride, (const bf16_t*)v,
                                                               v_stride, (const bf16_t*)v_first, vf_stride, lambda, G, hd, vd, eps,
-                                                              norm_dim, (bf16_t*)k_pages, (bf16_t*)v_pages, dest, PS, freqs, n_pairs, positions);
+                                                              norm_dim, (bf16_t*)k_pages, (bf16_t*)v_pages, dest, PS, freqs, n_pairs, positions, q_norm_w,
+                                                              k_norm_w, magnitude);
   return lev_check_launch("head_prepare_write");
 }
 
@@ -436,18 +445,20 @@ extern "C" int lev_poly_norm(const void* z, long z_stride, void* out, long o_str
 // o [T][H][NV][VD] (float32) holds, for every query head g and value head c, the attention weights of g applied to the
 // values of c. Head h of the result uses the values of its own value head c(h) = h / (H / KVH) with the weights of all
 // query heads mixed by `talk` [H][H]:   a[t][h][:] = gate(t, h) * sum_g talk[h][g] * o[t][g][c(h)][:].
-// talk == null: NV is 1 and the sum is o[t][h][0][:]. gate == null: 1, else sigmoid of the gate's entry. Everything is
-// multiplied by out_scale (a branch's weight in a sum of branches; 1 otherwise).
+// talk == null: NV is 1 and the sum is o[t][h][0][:]. gate == null: 1, else sigmoid of the gate's entry: one per (token, head),
+// or with gate_elements one per (token, head, element), laid out like the result. Everything is multiplied by out_scale (a
+// branch's weight in a sum of branches; 1 otherwise).
 template <typename T>
 __global__ void __launch_bounds__(64)
 head_talk_kernel(const float* __restrict__ o, const float* __restrict__ talk, const T* __restrict__ gate, long g_stride,
-                 T* __restrict__ a, long a_stride, int H, int KVH, int NV, int VD, float out_scale) {
+                 T* __restrict__ a, long a_stride, int H, int KVH, int NV, int VD, float out_scale, int gate_elements) {
   const int t = blockIdx.x, h = blockIdx.y;
   const float* ot = o + (size_t)t * H * NV * VD;
   const int c = talk ? h / (H / KVH) : 0;
   float gv = out_scale;
-  if (gate) gv = out_scale / (1.0f + expf(-to_float<T>(gate[(size_t)t * g_stride + h])));
+  if (gate && !gate_elements) gv = out_scale / (1.0f + expf(-to_float<T>(gate[(size_t)t * g_stride + h])));
   for (int d = threadIdx.x; d < VD; d += 64) {
+    if (gate && gate_elements) gv = out_scale / (1.0f + expf(-to_float<T>(gate[(size_t)t * g_stride + (size_t)h * VD + d])));
     float s;
     if (talk) {
       s = 0.f;
@@ -461,16 +472,16 @@ head_talk_kernel(const float* __restrict__ o, const float* __restrict__ talk, co
 }
 
 extern "C" int lev_head_talk(const float* o, const float* talk, const void* gate, long g_stride, void* a, long a_stride, int T, int H,
-                             int KVH, int NV, int VD, float out_scale, int dtype, hipStream_t stream) {
+                             int KVH, int NV, int VD, float out_scale, int gate_elements, int dtype, hipStream_t stream) {
   LEV_REQUIRE(T >= 0 && H > 0 && KVH > 0 && H % KVH == 0 && VD > 0, "head_talk: bad sizes T=%d heads=%d kv_heads=%d vd=%d", T, H, KVH, VD);
   LEV_REQUIRE(NV == (talk ? KVH : 1), "head_talk: %d outputs per query head; with a mixing matrix there are kv_heads=%d, without it one", NV, KVH);
   LEV_REQUIRE(a_stride >= (long)H * VD && H <= 65535, "head_talk: the output's row stride is too small, or too many heads");
   LEV_REQUIRE(dtype == LEV_F32 || dtype == LEV_BF16, "head_talk: unknown dtype %d", dtype);
   if (T == 0) return 0;
   if (dtype == LEV_F32)
-    head_talk_kernel<float><<<dim3(T, H), 64, 0, stream>>>(o, talk, (const float*)gate, g_stride, (float*)a, a_stride, H, KVH, NV, VD, out_scale);
+    head_talk_kernel<float><<<dim3(T, H), 64, 0, stream>>>(o, talk, (const float*)gate, g_stride, (float*)a, a_stride, H, KVH, NV, VD, out_scale, gate_elements);
   else
-    head_talk_kernel<bf16_t><<<dim3(T, H), 64, 0, stream>>>(o, talk, (const bf16_t*)gate, g_stride, (bf16_t*)a, a_stride, H, KVH, NV, VD, out_scale);
+    head_talk_kernel<bf16_t><<<dim3(T, H), 64, 0, stream>>>(o, talk, (const bf16_t*)gate, g_stride, (bf16_t*)a, a_stride, H, KVH, NV, VD, out_scale, gate_elements);
   return lev_check_launch("head_talk");
 }
 
@@ -583,4 +594,58 @@ extern "C" int lev_norm_average(float* streams, float* x, const float* w, int n,
   else
     norm_average_kernel<bf16_t, 256><<<n_rows, 256, lds, stream>>>(streams, x, w, n, count, norm_weight, (bf16_t*)out, rows, D, eps, vec);
   return lev_check_launch("norm_average");
+}
+
+// ------------------------------------------------------------------------------------------
+// The activation of a gated feed-forward between its two products: a row of z holds F gate sums and then F up sums,
+//     out[f] = act(g) * (u + up_shift),   g = z[f], u = z[F + f];   with limit > 0: g = min(g, limit), u = clamp(u, -limit, limit).
+// 32-bit arithmetic; `out` may be the first F columns of `z` (a thread reads both of its inputs before it writes).
+template <typename T>
+__global__ void __launch_bounds__(256)
+glu_activate_kernel(const T* __restrict__ z, long z_stride, T* __restrict__ out, long o_stride, int F, int act, float limit, float up_shift) {
+  const int t = blockIdx.x;
+  for (int f = threadIdx.x; f < F; f += 256) {
+    float g = to_float<T>(z[(size_t)t * z_stride + f]), u = to_float<T>(z[(size_t)t * z_stride + F + f]);
+    if (limit > 0.f) g = fminf(g, limit), u = fminf(fmaxf(u, -limit), limit);
+    out[(size_t)t * o_stride + f] = from_float<T>(lev_activate(g, act) * (u + up_shift));
+  }
+}
+
+extern "C" int lev_glu_activate(const void* z, long z_stride, void* out, long o_stride, int T, int F, int act, float limit, float up_shift, int dtype,
+                                hipStream_t stream) {
+  LEV_REQUIRE(T >= 0 && F > 0 && z && out && z_stride >= 2L * F && o_stride >= F, "glu_activate: bad sizes T=%d F=%d", T, F);
+  LEV_REQUIRE(act >= 0 && act <= LEV_ACT_LAST && limit >= 0.f, "glu_activate: unknown activation %d or a negative limit", act);
+  LEV_REQUIRE(dtype == LEV_F32 || dtype == LEV_BF16, "glu_activate: unknown dtype %d", dtype);
+  if (T == 0) return 0;
+  if (dtype == LEV_F32) glu_activate_kernel<float><<<T, 256, 0, stream>>>((const float*)z, z_stride, (float*)out, o_stride, F, act, limit, up_shift);
+  else glu_activate_kernel<bf16_t><<<T, 256, 0, stream>>>((const bf16_t*)z, z_stride, (bf16_t*)out, o_stride, F, act, limit, up_shift);
+  return lev_check_launch("glu_activate");
+}
+
+// ------------------------------------------------------------------------------------------
+// The sum of two branches that each pass an RMS norm of their own first: y = sa * a / rms(a) * wa + sb * b / rms(b) * wb over rows
+// of D float32 numbers, rms(v) = sqrt(mean(v^2) + eps). One workgroup per row; `y` may be `a` or `b`.
+__global__ void __launch_bounds__(256)
+norm_sum2_kernel(const float* __restrict__ a, const float* __restrict__ b, const float* __restrict__ wa, const float* __restrict__ wb, float sa,
+                 float sb, float eps, float* __restrict__ y, int D) {
+  __shared__ float red[8];
+  const size_t row = (size_t)blockIdx.x * D;
+  float ssa = 0.f, ssb = 0.f;
+  for (int d = threadIdx.x; d < D; d += 256) {
+    const float av = a[row + d], bv = b[row + d];
+    ssa = fmaf(av, av, ssa);
+    ssb = fmaf(bv, bv, ssb);
+  }
+  ssa = block_sum<256>(ssa, red);
+  ssb = block_sum<256>(ssb, red);
+  const float ra = sa / sqrtf(ssa / (float)D + eps), rb = sb / sqrtf(ssb / (float)D + eps);
+  for (int d = threadIdx.x; d < D; d += 256) y[row + d] = a[row + d] * ra * wa[d] + b[row + d] * rb * wb[d];
+}
+
+extern "C" int lev_norm_sum2(const float* a, const float* b, const float* wa, const float* wb, float sa, float sb, float eps, float* y, int T, int D,
+                             hipStream_t stream) {
+  LEV_REQUIRE(T >= 0 && D > 0 && a && b && wa && wb && y, "norm_sum2: a tensor is missing or bad sizes T=%d D=%d", T, D);
+  if (T == 0) return 0;
+  norm_sum2_kernel<<<T, 256, 0, stream>>>(a, b, wa, wb, sa, sb, eps, y, D);
+  return lev_check_launch("norm_sum2");
 }

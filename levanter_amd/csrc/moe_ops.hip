@@ -1,7 +1,8 @@
 // A feed-forward made of many small experts of which every token uses a few (a mixture of experts), steered from the device:
 // no count ever goes to the host, so the launches depend on the number of tokens alone.
 //
-//   route     per token: scores s = sigmoid(z) of the router's logits z (float32 [T][E]); the choice goes by c = s + correction;
+//   route     per token: scores s = sigmoid(z) of the router's logits z (float32 [T][E]), or with `softmax` the softmax of z over all
+//             E outputs; the choice goes by c = s + correction;
 //             the experts form G equal groups of neighbours, a group's score is the sum of its `group_top` largest c, only the
 //             experts of the `keep` best groups can be chosen (the others count as -inf); the `top` largest c win (ties: the
 //             lower index); the weights are the winners' s (times 1 / their sum if `renormalize`), in the order of falling c.
@@ -14,7 +15,11 @@
 //             bfloat16 on the matrix cores (16x16x32): few tiles of 16 rows with K split over a workgroup's waves, many with a
 //             wave per tile, tiles of 64 rows with both operands staged through LDS; float32 in plain arithmetic. Workgroups
 //             beyond n_tiles return at once.
+//             with limit > 0 the gate sum is capped at limit and the up sum clamped to +-limit first, and up_shift is added to
+//             the up sum: act(min(gate, limit)) * (clamp(up) + up_shift).
 //   combine   y[t] = sum_c weight[t][c] * out[pos_of[t * top + c]], c in order, float32; with `accumulate` added to what y holds.
+//   identity  router outputs n_real .. E-1 may stand for experts without weights whose result is their input: sort gives their pairs
+//             places but no tiles (the products never see them), and combine takes the token's own row of `identity_in` for them.
 #include "common.h"
 
 #define MOE_TM 16          // rows of a matrix-core row tile; a tile of the list has tile_rows = MOE_TM or 4 * MOE_TM rows
@@ -24,13 +29,23 @@
 // ---- route ------------------------------------------------------------------------------------
 __global__ void __launch_bounds__(64)
 moe_route_kernel(const float* __restrict__ z, long z_stride, const float* __restrict__ correction, int E, int G, int keep, int group_top, int top,
-                 int renormalize, int* __restrict__ chosen, float* __restrict__ weights) {
+                 int renormalize, int softmax, int* __restrict__ chosen, float* __restrict__ weights) {
   __shared__ float s_s[MOE_MAX_E], c_s[MOE_MAX_E], g_s[MOE_MAX_E];
   __shared__ int sel[MOE_MAX_TOP];
   const int t = blockIdx.x, lane = threadIdx.x;
   const int per = E / G;
+  float z_max = 0.f, inv_sum = 1.0f;
+  if (softmax) {
+    float mx = -INFINITY;
+    for (int e = lane; e < E; e += 64) mx = fmaxf(mx, z[(size_t)t * z_stride + e]);
+    z_max = wave_max(mx);
+    float sum = 0.f;
+    for (int e = lane; e < E; e += 64) sum += expf(z[(size_t)t * z_stride + e] - z_max);
+    inv_sum = 1.0f / wave_sum(sum);
+  }
   for (int e = lane; e < E; e += 64) {
-    const float s = 1.0f / (1.0f + expf(-z[(size_t)t * z_stride + e]));
+    const float ze = z[(size_t)t * z_stride + e];
+    const float s = softmax ? expf(ze - z_max) * inv_sum : 1.0f / (1.0f + expf(-ze));
     s_s[e] = s;
     c_s[e] = s + (correction ? correction[e] : 0.f);
   }
@@ -92,13 +107,13 @@ moe_route_kernel(const float* __restrict__ z, long z_stride, const float* __rest
 }
 
 extern "C" int lev_moe_route(const float* z, long z_stride, const float* correction, int T, int E, int G, int keep, int group_top, int top,
-                             int renormalize, int* chosen, float* weights, hipStream_t stream) {
+                             int renormalize, int softmax, int* chosen, float* weights, hipStream_t stream) {
   LEV_REQUIRE(T >= 0 && E > 0 && E <= MOE_MAX_E, "experts: %d experts (at most %d)", E, MOE_MAX_E);
   LEV_REQUIRE(G > 0 && E % G == 0 && keep > 0 && keep <= G && group_top > 0, "experts: %d groups of %d experts, %d kept", G, E, keep);
   LEV_REQUIRE(top > 0 && top <= MOE_MAX_TOP && top <= keep * (E / G), "experts: %d experts a token out of %d that can be chosen (at most %d)", top, keep * (E / G), MOE_MAX_TOP);
   LEV_REQUIRE(z && chosen && weights && z_stride >= E, "experts: a tensor is missing");
   if (T == 0) return 0;
-  moe_route_kernel<<<T, 64, 0, stream>>>(z, z_stride, correction, E, G, keep, group_top, top, renormalize, chosen, weights);
+  moe_route_kernel<<<T, 64, 0, stream>>>(z, z_stride, correction, E, G, keep, group_top, top, renormalize, softmax, chosen, weights);
   return lev_check_launch("moe_route");
 }
 
@@ -107,7 +122,7 @@ extern "C" int lev_moe_route(const float* z, long z_stride, const float* correct
 // themselves is whatever the atomic counters give: a pair's results do not depend on its place in a tile.
 #define MOE_SORT_NT 1024
 __global__ void __launch_bounds__(MOE_SORT_NT)
-moe_sort_kernel(const int* __restrict__ chosen, int P, int E, int tile_rows, int* __restrict__ sorted, int* __restrict__ pos_of,
+moe_sort_kernel(const int* __restrict__ chosen, int P, int E, int n_real, int tile_rows, int* __restrict__ sorted, int* __restrict__ pos_of,
                 int* __restrict__ tiles, int* __restrict__ meta) {
   __shared__ int count[MOE_MAX_E], start[MOE_MAX_E], tile_start[MOE_MAX_E + 1], cursor[MOE_MAX_E];
   const int tid = threadIdx.x;
@@ -121,7 +136,7 @@ moe_sort_kernel(const int* __restrict__ chosen, int P, int E, int tile_rows, int
       start[e] = at;
       tile_start[e] = tile;
       at += count[e];
-      tile += (count[e] + tile_rows - 1) / tile_rows;
+      if (e < n_real) tile += (count[e] + tile_rows - 1) / tile_rows;  // experts without weights get places and no tiles
     }
     tile_start[E] = tile;
     meta[0] = tile;
@@ -146,23 +161,27 @@ moe_sort_kernel(const int* __restrict__ chosen, int P, int E, int tile_rows, int
 
 extern "C" int lev_moe_max_tiles(int P, int E, int tile_rows) { return P / tile_rows + E + 1; }
 
-extern "C" int lev_moe_sort(const int* chosen, int P, int E, int tile_rows, int* sorted, int* pos_of, int* tiles, int* meta, hipStream_t stream) {
+extern "C" int lev_moe_sort(const int* chosen, int P, int E, int n_real, int tile_rows, int* sorted, int* pos_of, int* tiles, int* meta, hipStream_t stream) {
   LEV_REQUIRE(P >= 0 && E > 0 && E <= MOE_MAX_E, "experts: %d experts (at most %d)", E, MOE_MAX_E);
   LEV_REQUIRE(tile_rows == MOE_TM || tile_rows == 4 * MOE_TM, "experts: tiles of %d rows (%d or %d)", tile_rows, MOE_TM, 4 * MOE_TM);
   LEV_REQUIRE(chosen && sorted && pos_of && tiles && meta, "experts: a tensor is missing");
-  moe_sort_kernel<<<1, MOE_SORT_NT, 0, stream>>>(chosen, P, E, tile_rows, sorted, pos_of, tiles, meta);
+  LEV_REQUIRE(n_real >= 0 && n_real <= E, "experts: %d of %d experts have weights", n_real, E);
+  moe_sort_kernel<<<1, MOE_SORT_NT, 0, stream>>>(chosen, P, E, n_real, tile_rows, sorted, pos_of, tiles, meta);
   return lev_check_launch("moe_sort");
 }
 
 // ---- the experts' products ------------------------------------------------------------------------
-__device__ __forceinline__ float moe_act(float gate, float up, int act) { return lev_activate(gate, act) * up; }
+__device__ __forceinline__ float moe_act(float gate, float up, int act, float limit, float up_shift) {
+  if (limit > 0.f) gate = fminf(gate, limit), up = fminf(fmaxf(up, -limit), limit);
+  return lev_activate(gate, act) * (up + up_shift);
+}
 
 // float32: a thread per (row of the tile, output); 16 x 16 a workgroup
 template <typename T, typename TO>
 __global__ void __launch_bounds__(256)
 moe_linear_plain_kernel(const T* __restrict__ a, long a_stride, const T* __restrict__ w, TO* __restrict__ out, long o_stride,
                         const int* __restrict__ tiles, const int* __restrict__ meta, const int* __restrict__ sorted, int top, int gather,
-                        int K, int N, int F, int glu, int act) {
+                        int K, int N, int F, int glu, int act, float limit, float up_shift) {
   const int tile = blockIdx.x;
   if (tile >= meta[0]) return;
   const int e = tiles[3 * tile], first = tiles[3 * tile + 1], rows = tiles[3 * tile + 2];
@@ -177,7 +196,7 @@ moe_linear_plain_kernel(const T* __restrict__ a, long a_stride, const T* __restr
     if (glu) {
       const T* wu = wg + (size_t)F * K;
       for (int kk = 0; kk < K; ++kk) acc_up = fmaf(to_float<T>(wu[kk]), to_float<T>(ar[kk]), acc_up);
-      acc = moe_act(acc, acc_up, act);
+      acc = moe_act(acc, acc_up, act, limit, up_shift);
     }
     out[(size_t)pos * o_stride + o] = from_float<TO>(acc);
   }
@@ -199,7 +218,7 @@ template <typename TO, int NT, bool GLU, int RT>
 __global__ void __launch_bounds__(256)
 moe_linear_mfma_kernel(const bf16_t* __restrict__ a, long a_stride, const bf16_t* __restrict__ w, TO* __restrict__ out, long o_stride,
                        const int* __restrict__ tiles, const int* __restrict__ meta, const int* __restrict__ sorted, int top, int gather,
-                       int K, int N, int F, int act) {
+                       int K, int N, int F, int act, float limit, float up_shift) {
   const int tile = blockIdx.x;
   if (tile >= meta[0]) return;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, col = lane & 15, g = lane >> 4;
@@ -254,7 +273,7 @@ moe_linear_mfma_kernel(const bf16_t* __restrict__ a, long a_stride, const bf16_t
       for (int r = 0; r < 4; ++r) {
         const int o = o0 + 16 * nt + 4 * g + r;
         if (o < F)
-          out[(size_t)(first + 16 * rt + col) * o_stride + o] = from_float<TO>(GLU ? moe_act(acc[rt][nt][r], acc_up[rt][nt][r], act) : acc[rt][nt][r]);
+          out[(size_t)(first + 16 * rt + col) * o_stride + o] = from_float<TO>(GLU ? moe_act(acc[rt][nt][r], acc_up[rt][nt][r], act, limit, up_shift) : acc[rt][nt][r]);
       }
   }
 }
@@ -267,7 +286,7 @@ template <typename TO, bool GLU>
 __global__ void __launch_bounds__(64 * MOE_KS)
 moe_linear_splitk_kernel(const bf16_t* __restrict__ a, long a_stride, const bf16_t* __restrict__ w, TO* __restrict__ out, long o_stride,
                          const int* __restrict__ tiles, const int* __restrict__ meta, const int* __restrict__ sorted, int top, int gather,
-                         int K, int N, int F, int act) {
+                         int K, int N, int F, int act, float limit, float up_shift) {
   __shared__ float part[MOE_KS][2][4][64];
   const int tile = blockIdx.x;
   if (tile >= meta[0]) return;
@@ -309,7 +328,7 @@ moe_linear_splitk_kernel(const bf16_t* __restrict__ a, long a_stride, const bf16
       if (GLU) sum_up += part[q][1][r][lane];
     }
     const int o = o0 + 4 * g + r;
-    if (o < F) out[(size_t)(first + col) * o_stride + o] = from_float<TO>(GLU ? moe_act(sum, sum_up, act) : sum);
+    if (o < F) out[(size_t)(first + col) * o_stride + o] = from_float<TO>(GLU ? moe_act(sum, sum_up, act, limit, up_shift) : sum);
   }
 }
 
@@ -323,7 +342,7 @@ template <typename TO, bool GLU>
 __global__ void __launch_bounds__(256)
 moe_linear_tile_kernel(const bf16_t* __restrict__ a, long a_stride, const bf16_t* __restrict__ w, TO* __restrict__ out, long o_stride,
                        const int* __restrict__ tiles, const int* __restrict__ meta, const int* __restrict__ sorted, int top, int gather,
-                       int K, int N, int F, int act) {
+                       int K, int N, int F, int act, float limit, float up_shift) {
   constexpr int WR = GLU ? 2 * MOE_BN : MOE_BN, WL = WR / 64;  // weight rows of a workgroup, loads of them per thread and k-step
   __shared__ __attribute__((aligned(16))) bf16_t sa[2][64][MOE_LD];
   __shared__ __attribute__((aligned(16))) bf16_t sw[2][WR][MOE_LD];
@@ -397,15 +416,15 @@ moe_linear_tile_kernel(const bf16_t* __restrict__ a, long a_stride, const bf16_t
       for (int r = 0; r < 4; ++r) {
         const int o = o0 + wave * 32 + 16 * nt + 4 * g + r;
         if (o < F)
-          out[(size_t)(first + 16 * rt + col) * o_stride + o] = from_float<TO>(GLU ? moe_act(acc[rt][nt][r], acc_up[rt][nt][r], act) : acc[rt][nt][r]);
+          out[(size_t)(first + 16 * rt + col) * o_stride + o] = from_float<TO>(GLU ? moe_act(acc[rt][nt][r], acc_up[rt][nt][r], act, limit, up_shift) : acc[rt][nt][r]);
       }
   }
 }
 
 // a [rows][K]; w [E][N][K] with N = F outputs, or with glu N = 2F: gate rows then up rows; out [P][F]
 extern "C" int lev_moe_linear(const void* a, long a_stride, const void* w, void* out, long o_stride, const int* tiles, const int* meta,
-                              const int* sorted, int max_tiles, int tile_rows, int top, int gather, int K, int N, int glu, int act, int dtype,
-                              int out_dtype, int use_mfma, hipStream_t stream) {
+                              const int* sorted, int max_tiles, int tile_rows, int top, int gather, int K, int N, int glu, int act, float limit,
+                              float up_shift, int dtype, int out_dtype, int use_mfma, hipStream_t stream) {
   LEV_REQUIRE(a && w && out && tiles && meta && sorted, "experts: a tensor is missing");
   LEV_REQUIRE(K > 0 && N > 0 && (!glu || N % 2 == 0) && top > 0 && max_tiles >= 0, "experts: bad sizes K=%d N=%d", K, N);
   LEV_REQUIRE(act >= 0 && act <= LEV_ACT_LAST, "experts: unknown activation %d", act);
@@ -422,10 +441,10 @@ extern "C" int lev_moe_linear(const void* a, long a_stride, const void* w, void*
   do {                                                                                                                                           \
     if (glu)                                                                                                                                     \
       moe_linear_splitk_kernel<TO, true><<<grid_k, 64 * MOE_KS, 0, stream>>>((const bf16_t*)a, a_stride, (const bf16_t*)w, (TO*)out, o_stride, tiles, \
-                                                                            meta, sorted, top, gather, K, N, F, act);                            \
+                                                                            meta, sorted, top, gather, K, N, F, act, limit, up_shift);                            \
     else                                                                                                                                         \
       moe_linear_splitk_kernel<TO, false><<<grid_k, 64 * MOE_KS, 0, stream>>>((const bf16_t*)a, a_stride, (const bf16_t*)w, (TO*)out, o_stride, tiles, \
-                                                                             meta, sorted, top, gather, K, N, F, act);                           \
+                                                                             meta, sorted, top, gather, K, N, F, act, limit, up_shift);                           \
   } while (0)
       if (out_dtype == LEV_F32) MOE_SPLITK(float); else MOE_SPLITK(bf16_t);
 #undef MOE_SPLITK
@@ -437,10 +456,10 @@ extern "C" int lev_moe_linear(const void* a, long a_stride, const void* w, void*
   do {                                                                                                                                           \
     if (glu)                                                                                                                                     \
       moe_linear_tile_kernel<TO, true><<<grid_t, 256, 0, stream>>>((const bf16_t*)a, a_stride, (const bf16_t*)w, (TO*)out, o_stride, tiles, meta,   \
-                                                                  sorted, top, gather, K, N, F, act);                                            \
+                                                                  sorted, top, gather, K, N, F, act, limit, up_shift);                                            \
     else                                                                                                                                         \
       moe_linear_tile_kernel<TO, false><<<grid_t, 256, 0, stream>>>((const bf16_t*)a, a_stride, (const bf16_t*)w, (TO*)out, o_stride, tiles, meta,  \
-                                                                   sorted, top, gather, K, N, F, act);                                           \
+                                                                   sorted, top, gather, K, N, F, act, limit, up_shift);                                           \
   } while (0)
       if (out_dtype == LEV_F32) MOE_TILE(float); else MOE_TILE(bf16_t);
 #undef MOE_TILE
@@ -453,10 +472,10 @@ extern "C" int lev_moe_linear(const void* a, long a_stride, const void* w, void*
   do {                                                                                                                                           \
     if (glu)                                                                                                                                     \
       moe_linear_mfma_kernel<TO, 2, true, 1><<<grid, 256, 0, stream>>>((const bf16_t*)a, a_stride, (const bf16_t*)w, (TO*)out, o_stride, tiles, meta, \
-                                                                      sorted, top, gather, K, N, F, act);                                        \
+                                                                      sorted, top, gather, K, N, F, act, limit, up_shift);                                        \
     else                                                                                                                                         \
       moe_linear_mfma_kernel<TO, 2, false, 1><<<grid, 256, 0, stream>>>((const bf16_t*)a, a_stride, (const bf16_t*)w, (TO*)out, o_stride, tiles,  \
-                                                                       meta, sorted, top, gather, K, N, F, act);                                 \
+                                                                       meta, sorted, top, gather, K, N, F, act, limit, up_shift);                                 \
   } while (0)
     if (out_dtype == LEV_F32) MOE_CASE(float); else MOE_CASE(bf16_t);
 #undef MOE_CASE
@@ -465,39 +484,45 @@ extern "C" int lev_moe_linear(const void* a, long a_stride, const void* w, void*
   dim3 grid(max_tiles, (F + 15) / 16);
   if (dtype == LEV_F32)
     moe_linear_plain_kernel<float, float><<<grid, 256, 0, stream>>>((const float*)a, a_stride, (const float*)w, (float*)out, o_stride, tiles, meta,
-                                                                    sorted, top, gather, K, N, F, glu, act);
+                                                                    sorted, top, gather, K, N, F, glu, act, limit, up_shift);
   else if (out_dtype == LEV_F32)
     moe_linear_plain_kernel<bf16_t, float><<<grid, 256, 0, stream>>>((const bf16_t*)a, a_stride, (const bf16_t*)w, (float*)out, o_stride, tiles, meta,
-                                                                     sorted, top, gather, K, N, F, glu, act);
+                                                                     sorted, top, gather, K, N, F, glu, act, limit, up_shift);
   else
     moe_linear_plain_kernel<bf16_t, bf16_t><<<grid, 256, 0, stream>>>((const bf16_t*)a, a_stride, (const bf16_t*)w, (bf16_t*)out, o_stride, tiles,
-                                                                      meta, sorted, top, gather, K, N, F, glu, act);
+                                                                      meta, sorted, top, gather, K, N, F, glu, act, limit, up_shift);
   return lev_check_launch("moe_linear");
 }
 
 // ---- combine -------------------------------------------------------------------------------------
 __global__ void __launch_bounds__(256)
 moe_combine_kernel(const float* __restrict__ expert_out, const int* __restrict__ pos_of, const float* __restrict__ weights, float* __restrict__ y,
-                   int D, int top, int accumulate) {
+                   int D, int top, int accumulate, const int* __restrict__ chosen, int n_real, const void* __restrict__ identity_in, long id_stride,
+                   int id_dtype) {
   __shared__ int pos_s[MOE_MAX_TOP];
   __shared__ float w_s[MOE_MAX_TOP];
   const int t = blockIdx.x;
   if (threadIdx.x < top) {
-    pos_s[threadIdx.x] = pos_of[(size_t)t * top + threadIdx.x];
+    const bool own = identity_in != nullptr && chosen[(size_t)t * top + threadIdx.x] >= n_real;  // an expert that returns its input
+    pos_s[threadIdx.x] = own ? -1 : pos_of[(size_t)t * top + threadIdx.x];
     w_s[threadIdx.x] = weights[(size_t)t * top + threadIdx.x];
   }
   __syncthreads();
   for (int d = threadIdx.x; d < D; d += 256) {
     float acc = accumulate ? y[(size_t)t * D + d] : 0.f;
-    for (int c = 0; c < top; ++c) acc = fmaf(w_s[c], expert_out[(size_t)pos_s[c] * D + d], acc);
+    float own = 0.f;
+    if (identity_in != nullptr)
+      own = id_dtype == LEV_F32 ? ((const float*)identity_in)[(size_t)t * id_stride + d] : bf16_to_float(((const bf16_t*)identity_in)[(size_t)t * id_stride + d]);
+    for (int c = 0; c < top; ++c) acc = fmaf(w_s[c], pos_s[c] < 0 ? own : expert_out[(size_t)pos_s[c] * D + d], acc);
     y[(size_t)t * D + d] = acc;
   }
 }
 
 extern "C" int lev_moe_combine(const float* expert_out, const int* pos_of, const float* weights, float* y, int T, int D, int top, int accumulate,
-                               hipStream_t stream) {
+                               const int* chosen, int n_real, const void* identity_in, long id_stride, int id_dtype, hipStream_t stream) {
   LEV_REQUIRE(expert_out && pos_of && weights && y && T >= 0 && D > 0 && top > 0 && top <= MOE_MAX_TOP, "experts: bad arguments of the weighted sum");
+  LEV_REQUIRE(identity_in == nullptr || (chosen && id_stride >= D && (id_dtype == LEV_F32 || id_dtype == LEV_BF16)), "experts: experts that return their input need the choices and the input's rows");
   if (T == 0) return 0;
-  moe_combine_kernel<<<T, 256, 0, stream>>>(expert_out, pos_of, weights, y, D, top, accumulate);
+  moe_combine_kernel<<<T, 256, 0, stream>>>(expert_out, pos_of, weights, y, D, top, accumulate, chosen, n_real, identity_in, id_stride, id_dtype);
   return lev_check_launch("moe_combine");
 }

@@ -1,6 +1,6 @@
 // Rotary positions on queries and keys, in place, before the keys go to the cache. Pairs of neighbouring dimensions
 // (2i, 2i+1), i < n_pairs, of every head turn by the angle position * freqs[i]; dimensions from 2 * n_pairs on pass
-// unchanged:   (u, v) -> (u cos a - v sin a, v cos a + u sin a).
+// unchanged:   (u, v) -> (u cos a - v sin a, v cos a + u sin a). `magnitude` multiplies cosine and sine alike (1: a pure rotation).
 // Positions, angles, sine and cosine are 32-bit (sincosf with its full range reduction: an angle reaches thousands of
 // radians). freqs is a float32 table that the host makes from the base and whatever rescaling the model asks for.
 // One workgroup per token; its threads share the (head, pair) items of the query heads and then of the key heads.
@@ -9,7 +9,7 @@
 template <typename T>
 __global__ void __launch_bounds__(256)
 rotary_pairs_kernel(T* __restrict__ q, long q_stride, int HQ, T* __restrict__ k, long k_stride, int HK, int hd, int n_pairs,
-                    const float* __restrict__ freqs, const int* __restrict__ positions) {
+                    const float* __restrict__ freqs, const int* __restrict__ positions, float magnitude) {
   const int t = blockIdx.x;
   const float p = (float)positions[t];
   const int items = (HQ + HK) * n_pairs;
@@ -18,6 +18,7 @@ rotary_pairs_kernel(T* __restrict__ q, long q_stride, int HQ, T* __restrict__ k,
     T* row = head < HQ ? q + (size_t)t * q_stride + (size_t)head * hd : k + (size_t)t * k_stride + (size_t)(head - HQ) * hd;
     float s, c;
     sincosf(p * freqs[i], &s, &c);
+    s *= magnitude, c *= magnitude;
     const float u = to_float<T>(row[2 * i]), v = to_float<T>(row[2 * i + 1]);
     row[2 * i] = from_float<T>(u * c - v * s);
     row[2 * i + 1] = from_float<T>(v * c + u * s);
@@ -25,7 +26,7 @@ rotary_pairs_kernel(T* __restrict__ q, long q_stride, int HQ, T* __restrict__ k,
 }
 
 extern "C" int lev_rotary_pairs(void* q, long q_stride, int HQ, void* k, long k_stride, int HK, int hd, int n_pairs, const float* freqs,
-                                const int* positions, int T, int dtype, hipStream_t stream) {
+                                const int* positions, float magnitude, int T, int dtype, hipStream_t stream) {
   LEV_REQUIRE(T >= 0 && HQ >= 0 && HK >= 0 && hd > 0, "rotary: bad sizes T=%d heads=%d/%d head_dim=%d", T, HQ, HK, hd);
   LEV_REQUIRE(n_pairs >= 0 && 2 * n_pairs <= hd, "rotary: %d pairs do not fit a head of %d", n_pairs, hd);
   LEV_REQUIRE((HQ == 0 || q) && (HK == 0 || k) && freqs && positions, "rotary: a tensor is missing");
@@ -33,9 +34,9 @@ extern "C" int lev_rotary_pairs(void* q, long q_stride, int HQ, void* k, long k_
   LEV_REQUIRE(dtype == LEV_F32 || dtype == LEV_BF16, "rotary: unknown dtype %d", dtype);
   if (T == 0 || n_pairs == 0 || HQ + HK == 0) return 0;
   if (dtype == LEV_F32)
-    rotary_pairs_kernel<float><<<T, 256, 0, stream>>>((float*)q, q_stride, HQ, (float*)k, k_stride, HK, hd, n_pairs, freqs, positions);
+    rotary_pairs_kernel<float><<<T, 256, 0, stream>>>((float*)q, q_stride, HQ, (float*)k, k_stride, HK, hd, n_pairs, freqs, positions, magnitude);
   else
-    rotary_pairs_kernel<bf16_t><<<T, 256, 0, stream>>>((bf16_t*)q, q_stride, HQ, (bf16_t*)k, k_stride, HK, hd, n_pairs, freqs, positions);
+    rotary_pairs_kernel<bf16_t><<<T, 256, 0, stream>>>((bf16_t*)q, q_stride, HQ, (bf16_t*)k, k_stride, HK, hd, n_pairs, freqs, positions, magnitude);
   return lev_check_launch("rotary_pairs");
 }
 

@@ -92,7 +92,7 @@ def attention_values_unit(head_dim: int, value_dim: int) -> str:
         if head_dim % 16 or value_dim % 16 or not (16 <= head_dim <= 256 and 16 <= value_dim <= 256):
             raise ValueError(f"no matrix-core attention for head sizes {head_dim} / {value_dim}")
         register_unit(name, [("attention_values_mfma.hip", [f"-DLEV_HD={head_dim}", f"-DLEV_VD={value_dim}"], f"attention_values_mfma_hd{head_dim}_vd{value_dim}.o")],
-                      signatures={"lev_attention_values_mfma": [_P, _L, _P, _P, _P, _P, _P, _P, _I, _P, _I, _P, _I] + [_I] * 6 + [_F, _I, _I, _F, _P, _P, _I, _P, _I, _P],
+                      signatures={"lev_attention_values_mfma": [_P, _L, _P, _P, _P, _P, _P, _P, _I, _P, _I, _P, _I] + [_I] * 6 + [_F, _I, _I, _I, _F, _P, _P, _I, _P, _I, _P],
                                   "lev_attention_values_mfma_workspace": [_I, _I, _I, _I]})
     return name
 
@@ -272,21 +272,22 @@ _P, _I, _L, _F = ctypes.c_void_p, ctypes.c_int, ctypes.c_long, ctypes.c_float
 
 register_unit("core", ["errors.hip", "elementwise.hip", "layer_ops.hip", "gemm_simple.hip", "attention_simple.hip", "attention_values.hip",
                        "attention_common.hip", "stream_ops.hip", "rotary.hip", "block_linear.hip", "recurrent_ops.hip", "group_norm.hip", "delta_rule.hip",
-                       "moe_ops.hip"], signatures={
+                       "moe_ops.hip", "linear_attention.hip"], signatures={
     "lev_embed": [_P] * 5 + [_I, _I, _I, _F, _P],
+    "lev_pair_embed_add": [_P] * 6 + [_I, _I, _I, _L, _L, _I, _P],
     "lev_streams_step": [_P, _I, _I, _I, _P, _P, _P, _P, _P, _P, _F, _P, _P, _P, _I, _I, _P, _I, _P, _P],
-    "lev_rotary_pairs": [_P, _L, _I, _P, _L, _I, _I, _I, _P, _P, _I, _I, _P],
+    "lev_rotary_pairs": [_P, _L, _I, _P, _L, _I, _I, _I, _P, _P, _F, _I, _I, _P],
     "lev_latent_rope_write": [_P, _L, _I, _I, _I, _F, _P, _P, _L, _I, _I, _I, _I, _P, _P, _P, _P, _P, _I, _I, _I, _P],
     "lev_rotary_half": [_P, _L, _I, _I, _I, _I, _P, _P, _I, _I, _P],
     "lev_group_norm_step": [_P, _P, _P, _L, _I, _P, _F, _P, _P, _I, _P, _I, _I, _I, _F, _P],
     "lev_delta_rule": [_P] * 5 + [_L, _P, _L, _P, _P, _P, _P, _L, _I, _I, _I, _F, _F, _F, _I, _P],
     "lev_delta_rule_scan": [_P] * 5 + [_L, _P, _L, _P, _P, _P, _P, _L, _P, _I, _I, _I, _I, _F, _F, _F, _I, _P],
     "lev_delta_rule_scan_workspace": [_I, _I, _I],
-    "lev_moe_route": [_P, _L, _P] + [_I] * 7 + [_P, _P, _P],
+    "lev_moe_route": [_P, _L, _P] + [_I] * 8 + [_P, _P, _P],
     "lev_moe_max_tiles": [_I, _I, _I],
-    "lev_moe_sort": [_P, _I, _I, _I, _P, _P, _P, _P, _P],
-    "lev_moe_linear": [_P, _L, _P, _P, _L, _P, _P, _P] + [_I] * 11 + [_P],
-    "lev_moe_combine": [_P, _P, _P, _P, _I, _I, _I, _I, _P],
+    "lev_moe_sort": [_P, _I, _I, _I, _I, _P, _P, _P, _P, _P],
+    "lev_moe_linear": [_P, _L, _P, _P, _L, _P, _P, _P] + [_I] * 8 + [_F, _F, _I, _I, _I, _P],
+    "lev_moe_combine": [_P, _P, _P, _P, _I, _I, _I, _I, _P, _I, _P, _L, _I, _P],
     "lev_block_linear": [_P, _L, _P, _P, _P, _L] + [_I] * 7 + [_P],
     "lev_block_linear_mfma": [_P, _L, _P, _P, _P, _L] + [_I] * 6 + [_P],
     "lev_causal_conv": [_P, _L, _P, _P, _P, _P, _P, _L, _I, _I, _I, _I, _P],
@@ -297,14 +298,19 @@ register_unit("core", ["errors.hip", "elementwise.hip", "layer_ops.hip", "gemm_s
     "lev_norm_pending": [_P, _P, _I] + [_P] * 5 + [_I, _I, _I, _F, _I, _I, _P],
     "lev_kv_write": [_P, _P, _L, _L, _P, _P, _P] + [_I] * 6 + [_P],
     "lev_head_prepare": [_P, _L, _I, _I, _I, _F, _P, _L, _P, _L, _I, _I, _P, _P, _I, _I, _P],
-    "lev_head_prepare_write": [_P, _L, _I, _P, _L, _P, _L, _P, _L, _P, _I, _I, _I, _F, _I, _P, _P, _P, _I, _P, _I, _P, _I, _I, _P],
+    "lev_head_prepare_write": [_P, _L, _I, _P, _L, _P, _L, _P, _L, _P, _I, _I, _I, _F, _I, _P, _P, _P, _I, _P, _I, _P, _P, _P, _F, _I, _I, _P],
     "lev_norm_write_latent": [_P, _L, _I, _I, _F, _P, _P, _P, _P, _I, _I, _I, _P],
     "lev_recurrent_tokens": [_P, _L, _P, _L, _P, _P, _P, _P, _P, _P, _P, _P, _L, _I, _I, _I, _I, _F, _I, _P],
     "lev_poly_norm": [_P, _L, _P, _L, _P, _I, _I, _F, _I, _P],
-    "lev_head_talk": [_P, _P, _P, _L, _P, _L] + [_I] * 5 + [_F, _I, _P],
+    "lev_head_talk": [_P, _P, _P, _L, _P, _L] + [_I] * 5 + [_F, _I, _I, _P],
+    "lev_glu_activate": [_P, _L, _P, _L, _I, _I, _I, _F, _F, _I, _P],
+    "lev_norm_sum2": [_P, _P, _P, _P, _F, _F, _F, _P, _I, _I, _P],
+    "lev_gla_tokens": [_P, _P, _L, _P, _P, _L, _P, _L, _P, _P, _P, _P, _L, _I, _I, _I, _I, _F, _F, _F, _I, _I, _P],
+    "lev_gla_scan": [_P, _P, _L, _P, _P, _L, _P, _L, _P, _P, _P, _P, _L, _P, _I, _I, _I, _I, _I, _F, _F, _F, _I, _I, _P],
+    "lev_gla_scan_workspace": [_I, _I, _I, _I],
     "lev_stream_average": [_P, _P, _P, _I, _L, _P],
     "lev_norm_average": [_P, _P, _P, _I, _L, _P, _P, _P, _I, _I, _F, _I, _P],
-    "lev_attention_values": [_P, _L, _P, _P, _P, _P, _P, _P] + [_I] * 8 + [_F, _I, _I, _F, _P, _P, _I, _P],
+    "lev_attention_values": [_P, _L, _P, _P, _P, _P, _P, _P] + [_I] * 8 + [_F, _I, _I, _I, _F, _P, _P, _I, _P],
     "lev_sample": [_P, _L, _P, _P, _P, _P, _P, _P, _I, _I, _P],
     "lev_sample_workspace": [_I],
     "lev_feed_tokens": [_P, _P, _P, _I, _P],

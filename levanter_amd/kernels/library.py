@@ -225,6 +225,21 @@ class HipKernels:
         self._check(self.lib.lev_embed(_ptr(tokens), _ptr(positions), _ptr(table), _ptr(pos_table), _ptr(out), T, D,
                                        _DT[table.dtype], float(scale), self._s()))
 
+    def pair_embed_add(self, tokens, positions, token_slots, last_token, table, x, buckets: int, mul_prev: int, mul_cur: int) -> None:
+        """``x[t] += table[row]`` with ``row = (previous * mul_prev + tokens[t] * mul_cur) % buckets``, or row ``buckets`` (the table's
+        last) at position 0. The token before is the step's own token t - 1 where it belongs to the same request one position
+        earlier, else ``last_token[slot]`` (int32 ``[slots]``), which afterwards holds the last token of each request's run. Tokens
+        of nobody (slot < 0) take row ``buckets`` and store nothing."""
+        _dev(tokens, positions, token_slots, last_token, table, x)
+        T, D = x.shape
+        for t in (tokens, positions, token_slots):
+            _req(t.dtype == torch.int32 and t.numel() == T, "pair embedding: one int32 token, position and slot per row")
+        _req(last_token.dtype == torch.int32 and last_token.is_contiguous(), "pair embedding: the slots' last tokens must be int32")
+        _req(x.dtype == torch.float32 and x.is_contiguous(), "pair embedding: x must be contiguous float32")
+        _req(table.is_contiguous() and table.dtype in _DT and tuple(table.shape) == (buckets + 1, D), "pair embedding: the table must be [buckets + 1, D]")
+        self._check(self.lib.lev_pair_embed_add(_ptr(tokens), _ptr(positions), _ptr(token_slots), _ptr(last_token), _ptr(table), _ptr(x), T, D,
+                                                int(buckets), int(mul_prev), int(mul_cur), _DT[table.dtype], self._s()))
+
     def feed_tokens(self, dst, src, rows, n: int) -> None:
         """dst[i] = src[rows[i]] (``rows`` None: src[i]) for i < n: int32 token ids that never leave the device."""
         _dev(dst, src, rows)
@@ -462,12 +477,17 @@ class HipKernels:
 
     def head_prepare_write(self, q, k, v, k_pages, v_pages, dest, n_heads: int, n_kv_heads: int, head_dim: int, value_dim: int,
                            page_size: int, eps: Optional[float], v_first=None, blend=None, norm_dim: Optional[int] = None,
-                           rotary_freqs=None, positions=None) -> None:
+                           rotary_freqs=None, positions=None, q_norm_weight=None, k_norm_weight=None, rotary_magnitude: float = 1.0) -> None:
         """``head_prepare`` and ``kv_write`` in one kernel, for steps of single tokens: queries are normalised in place
         (``eps`` None: not at all), keys are normalised and values blended (``v_first`` None: not) on their way into the pages;
         ``k`` and ``v`` themselves stay as projected. ``rotary_freqs`` (float32, with ``positions``): the rotation of
-        ``rotary_pairs`` too, on the queries in place and on the keys on their way into the pages."""
-        _dev(q, k, v, k_pages, v_pages, dest, v_first, blend, rotary_freqs, positions)
+        ``rotary_pairs`` too (cosine and sine times ``rotary_magnitude``), on the queries in place and on the keys on their way into
+        the pages. ``q_norm_weight`` / ``k_norm_weight`` (float32 ``[head_dim]``): the normalised query / key heads are multiplied by
+        it, before the rotation."""
+        _dev(q, k, v, k_pages, v_pages, dest, v_first, blend, rotary_freqs, positions, q_norm_weight, k_norm_weight)
+        for w in (q_norm_weight, k_norm_weight):
+            _req(w is None or (eps is not None and w.dtype == torch.float32 and w.numel() == head_dim and w.is_contiguous()),
+                 "head_prepare_write: a norm's weight must be float32 [head_dim] and needs the norm")
         n_pairs = 0
         if rotary_freqs is not None:
             _req(rotary_freqs.dtype == torch.float32 and rotary_freqs.is_contiguous() and 2 * rotary_freqs.numel() <= head_dim, "head_prepare_write: float32 frequencies, at most head_dim / 2")
@@ -490,7 +510,8 @@ class HipKernels:
             _ptr(q), _rows(q, "head_prepare_write: q"), n_heads, _ptr(k), _rows(k, "head_prepare_write: k"), _ptr(v),
             _rows(v, "head_prepare_write: v"), _ptr(v_first), fs, _ptr(blend) if v_first is not None else None, n_kv_heads, head_dim,
             value_dim, float(eps or 0.0), int(norm_dim or head_dim) if eps is not None else 0, _ptr(k_pages), _ptr(v_pages), _ptr(dest), page_size,
-            _ptr(rotary_freqs) if n_pairs else None, n_pairs, _ptr(positions) if n_pairs else None, T, _DT[dt], self._s()))
+            _ptr(rotary_freqs) if n_pairs else None, n_pairs, _ptr(positions) if n_pairs else None, _ptr(q_norm_weight), _ptr(k_norm_weight),
+            float(rotary_magnitude), T, _DT[dt], self._s()))
 
     def norm_write_latent(self, c, weight, eps: float, norm_dim: int, k_pages, v_pages, dest, page_size: int) -> None:
         """``c`` ``[T, R]`` (one key/value head that all query heads share) becomes its RMS norm with ``weight`` (float32 ``[R]``;
@@ -560,10 +581,11 @@ class HipKernels:
         self._check(self.lib.lev_poly_norm(_ptr(z), _rows(z, "poly_norm: z"), _ptr(out), _rows(out, "poly_norm: out"), _ptr(coefficients),
                                            z.shape[0], z.shape[1], float(eps), _DT[z.dtype], self._s()))
 
-    def head_talk(self, o, talk, gate, out, n_heads: int, n_kv_heads: int, value_dim: int, out_scale: float = 1.0) -> None:
+    def head_talk(self, o, talk, gate, out, n_heads: int, n_kv_heads: int, value_dim: int, out_scale: float = 1.0, gate_elements: bool = False) -> None:
         """``o`` float32 [T, heads, NV, value_dim] (``attention_values``) -> ``out`` [T, heads*value_dim] in the compute dtype:
         head h gets ``sum_g talk[h, g] o[t, g, c(h)]`` with c(h) its own value head (``talk`` None: ``o[t, h, 0]``), times
-        ``sigmoid(gate[t, h])`` where ``gate`` [T, heads] (compute dtype) is given, times ``out_scale``."""
+        ``sigmoid(gate[t, h])`` where ``gate`` [T, heads] (compute dtype) is given (``gate_elements``: ``gate`` [T, heads*value_dim],
+        a gate per element of the result), times ``out_scale``."""
         _dev(o, talk, gate, out)
         T = out.shape[0]
         nv = n_kv_heads if talk is not None else 1
@@ -572,10 +594,10 @@ class HipKernels:
         _req(talk is None or (talk.dtype == torch.float32 and talk.shape == (n_heads, n_heads) and talk.is_contiguous()), "head_talk: the mixing matrix must be float32 [heads, heads]")
         gs = 0
         if gate is not None:
-            _req(gate.dtype == out.dtype and gate.shape == (T, n_heads), "head_talk: the gate must be [T, heads] of the compute dtype")
+            _req(gate.dtype == out.dtype and gate.shape == (T, n_heads * value_dim if gate_elements else n_heads), "head_talk: the gate must be [T, heads] (or [T, heads*value_dim]) of the compute dtype")
             gs = _rows(gate, "head_talk: gate")
         self._check(self.lib.lev_head_talk(_ptr(o), _ptr(talk), _ptr(gate), gs, _ptr(out), _rows(out, "head_talk: out"), T, n_heads, n_kv_heads,
-                                           nv, value_dim, float(out_scale), _DT[out.dtype], self._s()))
+                                           nv, value_dim, float(out_scale), int(bool(gate_elements) and gate is not None), _DT[out.dtype], self._s()))
 
     def stream_average(self, streams, x, weights, n: int, defer: bool = False) -> Optional[PendingAverage]:
         """``streams`` float32 [slots, T, D] holds earlier results in entries 0 .. n-2. ``x`` (float32 [T, D]) is kept as entry
@@ -592,12 +614,13 @@ class HipKernels:
 
     def attention_values(self, q, out, k_pages, v_pages, meta, *, n_heads: int, n_kv_heads: int, head_dim: int, value_dim: int,
                          all_value_heads: bool, page_size: int, scale: float, window: Optional[int], block_tables,
-                         softcap: Optional[float] = None, slopes=None, chunk: Optional[int] = None, sinks=None) -> None:
+                         softcap: Optional[float] = None, slopes=None, chunk: Optional[int] = None, sinks=None, keep_first: int = 0) -> None:
         """Causal attention over the pages for heads whose keys and values differ in size. ``out`` float32
         [T, heads, NV, value_dim]: the weights of each query head applied to the values of every key/value head
         (``all_value_heads``: NV = kv heads, for weights that are mixed over the heads afterwards, see ``head_talk``) or of its
         own (NV = 1). Score: ``cap(scale q.k) - slopes[h] * distance`` (``slopes`` float32 [heads] or None), ``cap`` the soft
         cap if given. ``chunk``: a query sees only the keys of its own chunk of that many positions, counted from position 0.
+        ``keep_first``: the first so many positions of a sequence stay in sight of every later query, whatever window and chunk say.
         ``sinks`` (float32 [heads] or None): the denominator of head h's softmax also holds ``exp(sinks[h])``, once per query.
         The cache must hold the step's own keys and values already."""
         _dev(q, out, k_pages, v_pages, block_tables, meta.positions, meta.token_seq, slopes, sinks)
@@ -618,7 +641,7 @@ class HipKernels:
             # single tokens: the keys of one token are split over several waves where the step's tokens alone leave the chip
             # empty (about 1,024 waves are aimed at, a block of 64 keys at least per wave); the step's description keeps the
             # choice and the scratch memory for all layers with these sizes
-            key = ("values", n_heads, n_kv_heads, value_dim, nv, int(window) if window else 0, int(chunk) if chunk else 0)
+            key = ("values", n_heads, n_kv_heads, value_dim, nv, int(window) if window else 0, int(chunk) if chunk else 0, int(keep_first))
             plan = meta.plans.get(key)
             if plan is None:
                 splits = 1
@@ -627,7 +650,7 @@ class HipKernels:
                     reach = min(int(window), meta.max_kv_len) if window else meta.max_kv_len
                     if chunk:
                         reach = min(reach, int(chunk))
-                    most = max(1, (reach + 63) // 64 + (1 if window or chunk else 0))
+                    most = max(1, (reach + 63) // 64 + (1 if window or chunk else 0) + ((int(keep_first) + 63) // 64 if window or chunk else 0))
                     splits = int(max(1, min(most, 32, 1024 // max(1, meta.n_decode * n_kv_heads * chunks))))
                 need = lib.lev_attention_values_mfma_workspace(meta.n_decode, splits, n_heads, nv) if splits > 1 else 0
                 ws = torch.empty(need, dtype=torch.uint8, device=q.device) if need else None
@@ -637,12 +660,12 @@ class HipKernels:
                 _ptr(q), _rows(q, "attention_values: q"), _ptr(out), _ptr(k_pages), _ptr(v_pages), _ptr(meta.positions), _ptr(meta.token_seq),
                 _ptr(block_tables), block_tables.shape[1], _ptr(meta.prefill_tiles), meta.n_prefill_tiles, _ptr(meta.decode_tokens),
                 meta.n_decode, n_heads, n_kv_heads, head_dim, value_dim, nv, page_size, float(scale), int(window) if window else 0,
-                int(chunk) if chunk else 0, float(softcap) if softcap else 0.0, _ptr(slopes), _ptr(sinks), splits, _ptr(ws), int(meta.max_kv_len), self._s()))
+                int(chunk) if chunk else 0, int(keep_first), float(softcap) if softcap else 0.0, _ptr(slopes), _ptr(sinks), splits, _ptr(ws), int(meta.max_kv_len), self._s()))
             return
         self._check(self.lib.lev_attention_values(
             _ptr(q), _rows(q, "attention_values: q"), _ptr(out), _ptr(k_pages), _ptr(v_pages), _ptr(meta.positions), _ptr(meta.token_seq),
             _ptr(block_tables), block_tables.shape[1], T, n_heads, n_kv_heads, head_dim, value_dim, nv, page_size, float(scale),
-            int(window) if window else 0, int(chunk) if chunk else 0, float(softcap) if softcap else 0.0, _ptr(slopes), _ptr(sinks), _DT[dt], self._s()))
+            int(window) if window else 0, int(chunk) if chunk else 0, int(keep_first), float(softcap) if softcap else 0.0, _ptr(slopes), _ptr(sinks), _DT[dt], self._s()))
 
     @staticmethod
     def mfma_attention_values_supports(head_dim: int, value_dim: int) -> bool:
@@ -688,9 +711,9 @@ class HipKernels:
         return None
 
     # ---- rotation of pairs ---------------------------------------------------------------------
-    def rotary_pairs(self, q, k, head_dim: int, freqs, positions) -> None:
+    def rotary_pairs(self, q, k, head_dim: int, freqs, positions, magnitude: float = 1.0) -> None:
         """In place on ``q`` ``[T, heads*head_dim]`` and ``k`` (either may be None): dimensions (2i, 2i+1) of every head turn by
-        ``positions[t] * freqs[i]``, i < len(freqs); the other dimensions stay. 32-bit angles."""
+        ``positions[t] * freqs[i]``, i < len(freqs), cosine and sine both times ``magnitude``; the other dimensions stay. 32-bit angles."""
         _dev(q, k, freqs, positions)
         ref = q if q is not None else k
         T, dt = ref.shape[0], ref.dtype
@@ -705,7 +728,7 @@ class HipKernels:
             _req(k.shape[0] == T and k.shape[1] % head_dim == 0, "rotary: k must be [T, heads*head_dim]")
             hk = k.shape[1] // head_dim
         self._check(self.lib.lev_rotary_pairs(_ptr(q), _rows(q, "rotary: q") if q is not None else 0, hq, _ptr(k), _rows(k, "rotary: k") if k is not None else 0,
-                                              hk, int(head_dim), freqs.numel(), _ptr(freqs), _ptr(positions), T, _DT[dt], self._s()))
+                                              hk, int(head_dim), freqs.numel(), _ptr(freqs), _ptr(positions), float(magnitude), T, _DT[dt], self._s()))
 
     # ---- block-diagonal products ---------------------------------------------------------------
     BLOCK_LINEAR_MAX_ROWS = 128  # plain arithmetic: more rows than this go block by block to the matrix products (a launch per block)
@@ -785,12 +808,13 @@ class HipKernels:
 
     # ---- norms in groups around gated sublayers ------------------------------------------------
     def group_norm_step(self, x, *, groups: int, eps: float, y=None, gate=None, post_weight=None, mult: float = 1.0, weight=None, h_out=None,
-                        rows=None, defer: bool = False, pending: Optional[PendingGatedNorm] = None) -> Optional[PendingGatedNorm]:
+                        rows=None, defer: bool = False, pending: Optional[PendingGatedNorm] = None, plain_read: bool = False) -> Optional[PendingGatedNorm]:
         """One pass over the rows of the residual stream ``x`` (float32 ``[T, D]``) with ``gn(v, w)`` = ``v`` split into ``groups``
         equal consecutive parts, each divided by its own ``sqrt(mean(part^2) + eps)``, times ``w``. In this order, whatever is
         given: the write of a sublayer's result, ``x <- x + mult * gn(y * sigmoid(gate), post_weight)`` (``y`` float32 ``[T, D]``;
         ``gate`` ``[T, D]`` float32 or compute dtype, rows may be strided, None: no gate); the read ``h_out = gn(x, weight)``
-        (compute dtype or float32). ``rows``: only these rows, into ``h_out [len(rows), D]``; ``x`` is not stored then.
+        (compute dtype or float32; ``plain_read``: ``h_out = x`` as it is, only rounded to ``h_out``'s type, for a sublayer that reads the
+        stream itself). ``rows``: only these rows, into ``h_out [len(rows), D]``; ``x`` is not stored then.
         ``defer``: nothing is launched; the write comes back as a ``PendingGatedNorm`` for the next call (``pending=``) or
         ``finish``. ``pending``: the write of an earlier call, done in this pass."""
         if pending is not None:
@@ -814,7 +838,7 @@ class HipKernels:
             _req(rows.dtype == torch.int32 and rows.is_contiguous() and h_out is not None, "group norm: rows must be int32 and need an output")
             n = rows.numel()
         if h_out is not None:
-            _req(weight is not None and h_out.dtype in _DT and h_out.is_contiguous() and tuple(h_out.shape) == (n, D), "group norm: bad normalised output")
+            _req((weight is not None) != bool(plain_read) and h_out.dtype in _DT and h_out.is_contiguous() and tuple(h_out.shape) == (n, D), "group norm: bad normalised output")
             odt = h_out.dtype
         self._check(self.lib.lev_group_norm_step(_ptr(x), _ptr(y), _ptr(gate), gs, _DT[gdt], _ptr(post_weight), float(mult), _ptr(weight), _ptr(h_out),
                                                  _DT[odt], _ptr(rows), n, D, int(groups), float(eps), self._s()))
@@ -868,9 +892,66 @@ class HipKernels:
                                             _ptr(norm_weight), _ptr(state), _ptr(token_slots), _ptr(out), _rows(out, "delta_rule: out"), T, n_heads,
                                             head_dim, float(norm_eps), float(key_eps), float(sharpness), _DT[dt], self._s()))
 
+    # ---- a matrix state per head that decays by key channel (gated linear attention) ------------
+    GLA_GATES = {"sigmoid": 0, "silu": 1}
+
+    def gated_linear_attention(self, q, k, v, g, z, norm_weight, state, token_slots, out, n_heads: int, key_dim: int, value_dim: int, tau: float,
+                               q_scale: float, norm_eps: float, gate: str = "silu", max_runs: Optional[int] = None) -> None:
+        """Per head, along each request's tokens, in 32-bit: ``a = sigmoid(z)^(1 / tau)``, ``S <- diag(a) S + k v^T``, ``o = S^T (q_scale q)``,
+        ``out = o / sqrt(mean(o^2) + norm_eps) * norm_weight * gate(g)`` (``gate``: "sigmoid", or "silu" = g sigmoid(g)). ``q, k``: ``[T, H*dk]``
+        views of one row stride, ``v, g``: ``[T, H*dv]`` views of one row stride, compute dtype; ``z`` float32 ``[T, H*dk]``; ``norm_weight``
+        float32 ``[H*dv]``; ``state`` float32 ``[slots, H, dk, dv]``, read and stored; ``token_slots`` int32 ``[T]`` (-1: a token of nobody,
+        zeros). ``max_runs``: the step has at most this many runs of consecutive tokens of one slot; given, and smaller than T, the step
+        takes the path for prompts."""
+        _dev(q, k, v, g, z, norm_weight, state, token_slots, out)
+        T = q.shape[0]
+        dt = q.dtype
+        H, dk, dv = int(n_heads), int(key_dim), int(value_dim)
+        _req(dt in _DT and tuple(q.shape) == tuple(k.shape) == (T, H * dk) and k.dtype == dt, "linear attention: q and k must be [T, heads*key_dim] of a compute dtype")
+        _req(tuple(v.shape) == tuple(g.shape) == (T, H * dv) and v.dtype == g.dtype == dt, "linear attention: v and g must be [T, heads*value_dim] of the same dtype")
+        qs, vs = _rows(q, "linear attention: q"), _rows(v, "linear attention: v")
+        _req(_rows(k, "linear attention: k") == qs and _rows(g, "linear attention: g") == vs, "linear attention: q and k, and v and g, must share a row stride")
+        _req(z.dtype == torch.float32 and tuple(z.shape) == (T, H * dk), "linear attention: z must be float32 [T, heads*key_dim]")
+        _req(norm_weight.dtype == torch.float32 and norm_weight.numel() == H * dv and norm_weight.is_contiguous(), "linear attention: the norm's weight must be float32 [heads*value_dim]")
+        _req(state.dtype == torch.float32 and state.is_contiguous() and tuple(state.shape[1:]) == (H, dk, dv), "linear attention: state must be float32 [slots, heads, dk, dv]")
+        _req(token_slots.dtype == torch.int32 and token_slots.numel() == T, "linear attention: one int32 slot per token")
+        _req(out.dtype == dt and tuple(out.shape) == (T, H * dv), "linear attention: out must be [T, heads*value_dim] of the compute dtype")
+        _req(gate in self.GLA_GATES, f"linear attention: unknown gate {gate!r}")
+        head = (_ptr(q), _ptr(k), qs, _ptr(v), _ptr(g), vs, _ptr(z), _rows(z, "linear attention: z"), _ptr(norm_weight), _ptr(state), _ptr(token_slots),
+                _ptr(out), _rows(out, "linear attention: out"))
+        tail = (H, dk, dv, float(tau), float(q_scale), float(norm_eps), self.GLA_GATES[gate], _DT[dt], self._s())
+        if max_runs is not None and max_runs < T:
+            ws = torch.empty(self.lib.lev_gla_scan_workspace(T, H, dk, dv) // 4, dtype=torch.float32, device=q.device)
+            self._check(self.lib.lev_gla_scan(*head, _ptr(ws), T, int(max_runs), *tail))
+            return
+        self._check(self.lib.lev_gla_tokens(*head, T, *tail))
+
+    # ---- row kernels of gated feed-forwards and of branches with norms of their own ---------------
+    def glu_activate(self, z, out, activation: str, limit: float = 0.0, up_shift: float = 0.0) -> None:
+        """``z`` ``[T, 2F]`` (gate sums, then up sums; rows may be strided) -> ``out`` ``[T, F]`` (may be ``z[:, :F]``):
+        ``act(g) * (u + up_shift)``, with ``limit`` > 0 after ``g = min(g, limit)``, ``u = clamp(u, -limit, limit)``. 32-bit arithmetic."""
+        _dev(z, out)
+        T, F2 = z.shape
+        _req(F2 % 2 == 0 and z.dtype in _DT and out.dtype == z.dtype and tuple(out.shape) == (T, F2 // 2), "glu_activate: z [T, 2F] and out [T, F] of one compute dtype")
+        _req(activation in ACTIVATIONS, f"glu_activate: unknown activation {activation!r}")
+        self._check(self.lib.lev_glu_activate(_ptr(z), _rows(z, "glu_activate: z"), _ptr(out), _rows(out, "glu_activate: out"), T, F2 // 2,
+                                              ACTIVATIONS[activation], float(limit), float(up_shift), _DT[z.dtype], self._s()))
+
+    def norm_sum2(self, a, b, weight_a, weight_b, scale_a: float, scale_b: float, eps: float, y) -> None:
+        """``y = scale_a * a / rms(a) * weight_a + scale_b * b / rms(b) * weight_b`` over rows, ``rms(v) = sqrt(mean(v^2) + eps)``; all
+        float32, ``y`` may be ``a`` or ``b``."""
+        _dev(a, b, weight_a, weight_b, y)
+        T, D = a.shape
+        for t in (a, b, y):
+            _req(t.dtype == torch.float32 and t.is_contiguous() and tuple(t.shape) == (T, D), "norm_sum2: contiguous float32 [T, D] tensors")
+        for w in (weight_a, weight_b):
+            _req(w.dtype == torch.float32 and w.is_contiguous() and w.numel() == D, "norm_sum2: the weights must be float32 [D]")
+        self._check(self.lib.lev_norm_sum2(_ptr(a), _ptr(b), _ptr(weight_a), _ptr(weight_b), float(scale_a), float(scale_b), float(eps), _ptr(y), T, D, self._s()))
+
     # ---- mixture of experts --------------------------------------------------------------------
-    def moe_route(self, z, correction, chosen, weights, *, n_groups: int = 1, keep: int = 1, group_top: int = 2, renormalize: bool = False) -> None:
-        """Per token: ``s = sigmoid(z)`` (``z`` float32 ``[T, E]``); the choice goes by ``s + correction``; only experts of the
+    def moe_route(self, z, correction, chosen, weights, *, n_groups: int = 1, keep: int = 1, group_top: int = 2, renormalize: bool = False,
+                  softmax: bool = False) -> None:
+        """Per token: ``s = sigmoid(z)`` (``z`` float32 ``[T, E]``), or with ``softmax`` the softmax of ``z`` over all E; the choice goes by ``s + correction``; only experts of the
         ``keep`` groups (of ``n_groups`` equal groups of neighbours) whose ``group_top`` largest choice scores sum highest can be
         chosen; ``chosen`` int32 ``[T, top]`` the winners in the order of falling choice score (ties: lower index first),
         ``weights`` float32 ``[T, top]`` their ``s`` (divided by their sum with ``renormalize``)."""
@@ -881,7 +962,7 @@ class HipKernels:
         _req(tuple(chosen.shape) == tuple(weights.shape) == (T, top) and chosen.is_contiguous() and weights.is_contiguous(), "experts: choices and weights must be [T, top]")
         _req(correction is None or (correction.dtype == torch.float32 and correction.numel() == E and correction.is_contiguous()), "experts: the correction must be float32 [E]")
         self._check(self.lib.lev_moe_route(_ptr(z), _rows(z, "experts: z"), _ptr(correction), T, E, int(n_groups), int(keep), int(group_top), top,
-                                           int(renormalize), _ptr(chosen), _ptr(weights), self._s()))
+                                           int(renormalize), int(bool(softmax)), _ptr(chosen), _ptr(weights), self._s()))
 
     @staticmethod
     def moe_tile_rows(pairs: int, n_experts: int) -> int:
@@ -891,21 +972,23 @@ class HipKernels:
     def moe_max_tiles(self, pairs: int, n_experts: int, tile_rows: int = 16) -> int:
         return int(self.lib.lev_moe_max_tiles(int(pairs), int(n_experts), int(tile_rows)))
 
-    def moe_sort(self, chosen, n_experts: int, sorted_pairs, pos_of, tiles, meta, tile_rows: int = 16) -> None:
+    def moe_sort(self, chosen, n_experts: int, sorted_pairs, pos_of, tiles, meta, tile_rows: int = 16, n_real: Optional[int] = None) -> None:
         """The (token, choice) pairs of ``chosen`` ordered by expert: ``sorted_pairs[pos]`` the pair at place ``pos``, ``pos_of`` its
         inverse, ``tiles`` int32 ``[max_tiles, 3]`` (expert, first place, rows <= ``tile_rows``) covering every expert's stretch,
-        ``meta[0]`` their number. Everything stays on the device."""
+        ``meta[0]`` their number. Everything stays on the device. ``n_real``: only the experts below it have weights; the pairs of the others
+        get places and no tiles (``moe_combine`` gives them the token's own input)."""
         _dev(chosen, sorted_pairs, pos_of, tiles, meta)
         P = chosen.numel()
         for t in (chosen, sorted_pairs, pos_of, tiles, meta):
             _req(t.dtype == torch.int32 and t.is_contiguous(), "experts: int32 tables")
         _req(sorted_pairs.numel() >= P and pos_of.numel() >= P and tiles.numel() >= 3 * self.moe_max_tiles(P, n_experts, tile_rows) and meta.numel() >= 1, "experts: tables too small")
-        self._check(self.lib.lev_moe_sort(_ptr(chosen), P, int(n_experts), int(tile_rows), _ptr(sorted_pairs), _ptr(pos_of), _ptr(tiles), _ptr(meta), self._s()))
+        self._check(self.lib.lev_moe_sort(_ptr(chosen), P, int(n_experts), int(n_experts if n_real is None else n_real), int(tile_rows), _ptr(sorted_pairs), _ptr(pos_of), _ptr(tiles), _ptr(meta), self._s()))
 
     def moe_linear(self, a, w, out, tiles, meta, sorted_pairs, *, top: int, gather: bool, glu: bool = False, activation: str = "none",
-                   tile_rows: int = 16) -> None:
+                   tile_rows: int = 16, limit: float = 0.0, up_shift: float = 0.0) -> None:
         """For every tile of ``moe_sort``: ``out[pos] = w[expert] a[row(pos)]``, ``row(pos)`` the pair's token (``gather``) or
-        ``pos`` itself. ``w`` ``[E, N, K]``; with ``glu`` N = 2F, gate rows then up rows, and ``out[pos][f] = act(gate_f) * up_f``."""
+        ``pos`` itself. ``w`` ``[E, N, K]``; with ``glu`` N = 2F, gate rows then up rows, and ``out[pos][f] = act(gate_f) * (up_f + up_shift)``;
+        with ``limit`` > 0 the gate sum is capped at it and the up sum clamped to +-limit first."""
         _dev(a, w, out, tiles, meta, sorted_pairs)
         _req(w.dim() == 3 and w.is_contiguous() and w.dtype in _DT and a.dtype == w.dtype and a.dim() == 2 and a.shape[1] == w.shape[2], "experts: a [rows, K], w [E, N, K] of one dtype")
         E, N, K = w.shape
@@ -913,17 +996,25 @@ class HipKernels:
         _req(out.dim() == 2 and out.shape[1] == F_ and out.dtype in _DT and (a.dtype == torch.bfloat16 or out.dtype == torch.float32), "experts: bad output")
         max_tiles = tiles.numel() // 3
         self._check(self.lib.lev_moe_linear(_ptr(a), _rows(a, "experts: a"), _ptr(w), _ptr(out), _rows(out, "experts: out"), _ptr(tiles), _ptr(meta),
-                                            _ptr(sorted_pairs), max_tiles, int(tile_rows), int(top), int(gather), K, N, int(glu), ACTIVATIONS[activation], _DT[a.dtype],
+                                            _ptr(sorted_pairs), max_tiles, int(tile_rows), int(top), int(gather), K, N, int(glu), ACTIVATIONS[activation], float(limit), float(up_shift), _DT[a.dtype],
                                             _DT[out.dtype], int(self.use_mfma), self._s()))
 
-    def moe_combine(self, expert_out, pos_of, weights, y, accumulate: bool = False) -> None:
-        """``y[t] = sum_c weights[t, c] * expert_out[pos_of[t, c]]``, c in order, float32; ``accumulate``: added to what ``y`` holds."""
-        _dev(expert_out, pos_of, weights, y)
+    def moe_combine(self, expert_out, pos_of, weights, y, accumulate: bool = False, chosen=None, n_real: int = 0, identity_in=None) -> None:
+        """``y[t] = sum_c weights[t, c] * expert_out[pos_of[t, c]]``, c in order, float32; ``accumulate``: added to what ``y`` holds.
+        ``identity_in`` (``[T, D]``, with ``chosen`` int32 ``[T, top]`` and ``n_real``): a choice of an expert from ``n_real`` on takes
+        ``identity_in[t]`` in place of an expert's output."""
+        _dev(expert_out, pos_of, weights, y, chosen, identity_in)
+        ids, idt = 0, torch.float32
+        if identity_in is not None:
+            _req(chosen is not None and chosen.dtype == torch.int32 and chosen.is_contiguous() and tuple(chosen.shape) == tuple(weights.shape)
+                 and identity_in.dtype in _DT and tuple(identity_in.shape) == tuple(y.shape), "experts: experts that return their input need the choices and the input")
+            ids, idt = _rows(identity_in, "experts: identity_in"), identity_in.dtype
         T, D = y.shape
         top = weights.shape[1]
         _req(expert_out.dtype == y.dtype == weights.dtype == torch.float32 and expert_out.is_contiguous() and y.is_contiguous() and weights.is_contiguous()
              and expert_out.shape[1] == D and expert_out.shape[0] >= T * top and pos_of.dtype == torch.int32 and pos_of.numel() >= T * top, "experts: bad arguments of the weighted sum")
-        self._check(self.lib.lev_moe_combine(_ptr(expert_out), _ptr(pos_of), _ptr(weights), _ptr(y), T, D, top, int(accumulate), self._s()))
+        self._check(self.lib.lev_moe_combine(_ptr(expert_out), _ptr(pos_of), _ptr(weights), _ptr(y), T, D, top, int(accumulate),
+                                             _ptr(chosen) if identity_in is not None else None, int(n_real), _ptr(identity_in), ids, _DT[idt], self._s()))
 
     # ---- attention -------------------------------------------------------------------------
     def paged_attention(self, q, out, k_pages, v_pages, meta, *, n_heads: int, n_kv_heads: int, head_dim: int,

@@ -1,5 +1,5 @@
 """Parts that layers are put together from. Importing the package registers the built-in kinds."""
-from . import (attention, block, delta_rule, embedding, feed_forward, gated_block, head, hyper_connections, latent_attention, moe, norm,  # noqa: F401
+from . import (attention, block, delta_rule, embedding, feed_forward, gated_block, head, hyper_connections, latent_attention, linear_attention, moe, norm,  # noqa: F401
                parallel_mixers, position, recurrent, stream_mix, talking_attention)
 from .base import (AttentionMeta, Block, BuildEnv, CacheUnitView, Embedding, FeedForward, GroupView, Head, Mixer, Norm, Part,
                    PositionEncoding, StepContext, StreamMix)

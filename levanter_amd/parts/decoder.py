@@ -69,7 +69,12 @@ class DecoderLm:
 
     def cache_requirements(self) -> List[Tuple[int, object]]:
         """(cache unit, requirement) of every unit that a plan entry writes."""
-        return [(e.cache, self.blocks[e.layer].cache_requirement()) for e in self.plan if e.writes_cache]
+        reqs = [(e.cache, self.blocks[e.layer].cache_requirement()) for e in self.plan if e.writes_cache]
+        own = getattr(self.embedding, "cache_requirement", None)
+        own = own() if own is not None else None
+        if own is not None:  # what the embedding keeps per request (a unit of its own, outside the plan's numbering)
+            reqs.append((self.embedding.STATE_UNIT, own))
+        return reqs
 
     def forward(self, ctx: StepContext, logit_rows: torch.Tensor) -> torch.Tensor:
         """Run the step's tokens through the plan; float32 logits ``[len(logit_rows), vocab]``."""

@@ -6,6 +6,7 @@ from typing import Dict, Optional
 
 import torch
 
+from levanter_amd.cache.requirements import SlotState
 from .base import BuildEnv, Embedding, StepContext
 from .registry import EMBEDDINGS, part_class
 from .spec import PartSpec
@@ -31,7 +32,13 @@ def tensors_of_nested(param: str, tensors: Dict[str, torch.Tensor]) -> Dict[str,
 class TokenEmbedding(Embedding):
     """params: ``vocab_size``, ``dim``, ``position`` (the description of a position encoding, or None), ``scale`` (a
     multiplier of the embedding's output, 1 by default), ``norm`` (the description of a norm that the residual stream's first
-    value goes through, or None; its class takes ``out_dtype`` and gives float32); tensor ``table``."""
+    value goes through, or None; its class takes ``out_dtype`` and gives float32), ``pairs`` (None, or ``{"buckets", "mul_prev",
+    "mul_cur"}``: the row ``(token before * mul_prev + token * mul_cur) mod buckets`` of ``pairs.table`` ``[buckets + 1, dim]`` is added, the
+    table's last row for a request's first token; the token before a step's first token is kept in the request's state slot); tensor
+    ``table``."""
+
+    STATE_UNIT = -1
+    """The cache unit of the embedding's own per-request state (the plan's entries count from 0)."""
 
     def __init__(self, spec: PartSpec, tensors: Dict[str, torch.Tensor], env: BuildEnv):
         super().__init__(spec, tensors, env)
@@ -43,6 +50,12 @@ class TokenEmbedding(Embedding):
         self.position = None
         if pos_spec is not None:
             self.position = part_class(pos_spec.kind, pos_spec.family or "position")(pos_spec, tensors_of_nested("position", tensors), env)
+        self.pairs = spec.params.get("pairs")
+        self.pair_table = None
+        if self.pairs is not None:
+            self.pair_table = tensors["pairs.table"].to(env.device, env.dtype).contiguous()
+            if tuple(self.pair_table.shape) != (int(self.pairs["buckets"]) + 1, self.dim):
+                raise ValueError(f"token_embedding: the pair table must be [{int(self.pairs['buckets']) + 1}, {self.dim}], got {list(self.pair_table.shape)}")
         norm_spec: Optional[PartSpec] = spec.params.get("norm")
         self.norm = None
         if norm_spec is not None:
@@ -56,6 +69,10 @@ class TokenEmbedding(Embedding):
     def max_positions(self) -> Optional[int]:
         return None if self.position is None else self.position.max_positions
 
+    def cache_requirement(self):
+        """What the embedding keeps per request between steps (None: nothing): the last token, for the pairs."""
+        return None if self.pairs is None else SlotState((1,), "int32")
+
     def __call__(self, ctx: StepContext) -> torch.Tensor:
         x = ctx.empty(ctx.n_tokens, self.dim, torch.float32)
         pos_table = None if self.position is None else self.position.embedding_table()
@@ -63,6 +80,10 @@ class TokenEmbedding(Embedding):
             ctx.kernels.embed(ctx.tokens, ctx.attention.positions, self.table, pos_table, x)
         else:
             ctx.kernels.embed(ctx.tokens, ctx.attention.positions, self.table, pos_table, x, scale=self.scale)
+        if self.pairs is not None:
+            last = ctx.units[self.STATE_UNIT].state.view(-1)
+            ctx.kernels.pair_embed_add(ctx.tokens, ctx.attention.positions, ctx.token_slots, last, self.pair_table, x,
+                                       int(self.pairs["buckets"]), int(self.pairs["mul_prev"]), int(self.pairs["mul_cur"]))
         if self.norm is not None:
             x = self.norm(x, ctx, out_dtype=torch.float32)
         return x

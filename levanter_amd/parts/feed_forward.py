@@ -37,6 +37,60 @@ class DenseMlp(FeedForward):
         self.down(self.up(h, ctx, activation=self.activation), ctx, out=y, may_leave=True)
 
 
+@FEED_FORWARDS.register("gated_mlp")
+class GatedMlp(FeedForward):
+    """down(act(gate h) * (up h + up_shift)): the two first products are one (gate rows, then up rows), the activation is a row
+    kernel in 32-bit between the products. With ``limit`` the gate's sums are capped at it and the up sums clamped to +-limit
+    before the activation. params: ``dim``, ``inner_dim``, ``activation``, ``limit`` (None), ``up_shift`` (0). Tensors ``[out, in]``:
+    ``gate.weight``, ``up.weight`` ``[inner, dim]``, ``down.weight`` ``[dim, inner]``, optional ``.bias`` of each. An inner width that
+    is no multiple of 8 carries zeros behind it."""
+
+    graph_safe = True
+
+    def __init__(self, spec: PartSpec, tensors: Dict[str, torch.Tensor], env: BuildEnv):
+        super().__init__(spec, tensors, env)
+        p = spec.params
+        self.activation = p["activation"]
+        if self.activation not in ACTIVATIONS:
+            raise ValueError(f"gated_mlp: unknown activation {self.activation!r}")
+        D, F = int(p["dim"]), int(p["inner_dim"])
+        self.limit = float(p["limit"]) if p.get("limit") else 0.0
+        self.up_shift = float(p.get("up_shift", 0.0))
+        Fp = self.inner_padded = (F + 7) // 8 * 8
+
+        def f32(name, shape):
+            t = tensors[name].to(torch.float32).cpu()
+            if tuple(t.shape) != tuple(shape):
+                raise ValueError(f"gated_mlp: {name} must be {list(shape)}, got {list(t.shape)}")
+            return t
+
+        w_in = torch.zeros(2 * Fp, D)
+        w_in[:F], w_in[Fp:Fp + F] = f32("gate.weight", (F, D)), f32("up.weight", (F, D))
+        b_in = None
+        if "gate.bias" in tensors or "up.bias" in tensors:
+            b_in = torch.zeros(2 * Fp)
+            if "gate.bias" in tensors:
+                b_in[:F] = f32("gate.bias", (F,))
+            if "up.bias" in tensors:
+                b_in[Fp:Fp + F] = f32("up.bias", (F,))
+        self.up = Linear(w_in, b_in, "out_in", env)
+        w_down = torch.zeros(D, Fp)
+        w_down[:, :F] = f32("down.weight", (D, F))
+        self.down = Linear(w_down, tensors.get("down.bias"), "out_in", env)
+
+    def _inner(self, h: torch.Tensor, ctx: StepContext) -> torch.Tensor:
+        z = self.up(h, ctx)
+        m = z[:, :self.inner_padded]
+        ctx.kernels.glu_activate(z, m, self.activation, limit=self.limit, up_shift=self.up_shift)
+        return m
+
+    def forward(self, h: torch.Tensor, x: torch.Tensor, ctx: StepContext) -> None:
+        self.down(self._inner(h, ctx), ctx, residual=x, final=True)
+
+    def compute(self, h: torch.Tensor, y: torch.Tensor, ctx: StepContext) -> None:
+        self.down(self._inner(h, ctx), ctx, out=y, may_leave=True)
+
+
 @FEED_FORWARDS.register("poly_norm_mlp")
 class PolyNormMlp(FeedForward):
     """down(act(up(h))) with an activation that needs a token's whole row: c0 N(z) + c1 N(z^2) + c2 N(z^3) + c3, powers

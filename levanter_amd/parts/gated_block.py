@@ -25,8 +25,8 @@ from .spec import PartSpec
 
 @NORMS.register("group_rmsnorm")
 class GroupRmsNorm(Norm):
-    """params: ``dim``, ``groups``, ``eps``; tensor ``weight`` ``[dim]``. Folds a pending gated write of the same grouping into
-    its pass."""
+    """params: ``dim``, ``groups``, ``eps``, ``weight_offset`` (0; 1 for a weight that is stored as its distance from one); tensor
+    ``weight`` ``[dim]``. Folds a pending gated write of the same grouping into its pass."""
 
     graph_safe = True
     folds_pending = True
@@ -36,7 +36,7 @@ class GroupRmsNorm(Norm):
         self.dim, self.groups, self.eps = int(spec.params["dim"]), int(spec.params["groups"]), float(spec.params["eps"])
         if self.dim % self.groups:
             raise ValueError(f"group_rmsnorm: {self.dim} numbers do not split into {self.groups} equal groups")
-        self.weight = tensors["weight"].to(env.device, torch.float32).contiguous()
+        self.weight = (tensors["weight"].to(env.device, torch.float32) + float(spec.params.get("weight_offset", 0.0))).contiguous()
         if self.weight.numel() != self.dim:
             raise ValueError(f"group_rmsnorm: the weight must have {self.dim} entries, got {self.weight.numel()}")
 
@@ -54,7 +54,8 @@ class GroupRmsNorm(Norm):
 @STREAM_MIXES.register("gated_post_norm")
 class GatedPostNorm(Part):
     """How one sublayer's result enters the residual stream: ``x <- x + mult * gn(y * sigmoid(gate.weight h + gate.bias), weight)``.
-    params: ``dim``, ``groups``, ``eps``, ``mult``, ``gate`` (False: no gate and no gate tensors). Tensors: ``weight`` ``[dim]``,
+    params: ``dim``, ``groups``, ``eps``, ``mult``, ``gate`` (False: no gate and no gate tensors), ``weight_offset`` (0; 1 for a weight
+    that is stored as its distance from one). Tensors: ``weight`` ``[dim]``,
     ``gate.weight`` ``[dim, dim]``, ``gate.bias`` ``[dim]``."""
 
     graph_safe = True
@@ -63,7 +64,7 @@ class GatedPostNorm(Part):
         super().__init__(spec, tensors, env)
         p = spec.params
         self.dim, self.groups, self.eps, self.mult = int(p["dim"]), int(p["groups"]), float(p["eps"]), float(p.get("mult", 1.0))
-        self.weight = tensors["weight"].to(env.device, torch.float32).contiguous()
+        self.weight = (tensors["weight"].to(env.device, torch.float32) + float(p.get("weight_offset", 0.0))).contiguous()
         self.gate = Linear(tensors["gate.weight"], tensors.get("gate.bias"), "out_in", env) if p.get("gate", True) else None
         if self.weight.numel() != self.dim or (self.gate is not None and (self.gate.n_in, self.gate.n_out) != (self.dim, self.dim)):
             raise ValueError("gated_post_norm: weights do not have the sizes of the description")
@@ -169,3 +170,54 @@ class GatedSandwichBlock(Block):
         self._sublayer(self.norm1, self.connect1, lambda h, y: self._run_mixer(h, y, ctx, unit, writes_cache), x, ctx)
         if self.feed_forward is not None:
             self._sublayer(self.norm2, self.connect2, lambda h, y: self._run_feed_forward(h, y, ctx), x, ctx)
+
+
+@BLOCKS.register("post_norm")
+class PostNormBlock(Block):
+    """Sublayers that read the residual stream itself and whose results are normed on their way into it:
+    ``x <- x + connect1(mixer(x))``, then (if the layer has one) ``x <- x + connect2(feed_forward(x))``; a ``connect`` is a
+    ``gated_post_norm`` (its gate may be switched off). There is no norm ahead of a sublayer: its input is the stream, rounded to
+    the compute dtype by the pass that also does the write of the sublayer before (one row kernel a sublayer)."""
+
+    roles = ("mixer", "connect1")
+    defers_residual = True  # the stream is read through that pass only
+
+    def __init__(self, parts: Dict[str, Part]):
+        super().__init__(parts)
+        unknown = [r for r in parts if r not in ("mixer", "connect1", "feed_forward", "connect2")]
+        if unknown:
+            raise ValueError(f"block 'post_norm' has no role {', '.join(unknown)}")
+        self.mixer, self.connect1 = parts["mixer"], parts["connect1"]
+        self.feed_forward: Optional[Part] = parts.get("feed_forward")
+        self.connect2 = parts.get("connect2")
+        if self.feed_forward is not None and self.connect2 is None:
+            raise ValueError("block 'post_norm': a feed-forward needs connect2")
+
+    @staticmethod
+    def _read(connect, x: torch.Tensor, ctx: StepContext) -> torch.Tensor:
+        """The stream as a sublayer's input; the write that the sublayer before has left pending is done in the same pass."""
+        pending = ctx.take_pending(x)
+        if pending is not None and not (isinstance(pending, PendingGatedNorm) and pending.groups == connect.groups and pending.eps == connect.eps):
+            ctx.kernels.finish(pending)
+            pending = None
+        h = ctx.empty(x.shape[0], x.shape[1])
+        ctx.kernels.group_norm_step(x, groups=connect.groups, eps=connect.eps, h_out=h, pending=pending, plain_read=True)
+        return h
+
+    def _sublayer(self, connect, run, x: torch.Tensor, ctx: StepContext) -> None:
+        may_defer = ctx.may_defer
+        h = self._read(connect, x, ctx)
+        y = torch.empty_like(x)
+        ctx.may_defer = False  # a sublayer's result is complete before it is normed
+        run(h, y)
+        product = ctx.take_product_pending(y)
+        if product is not None:
+            ctx.kernels.finish(product)
+        gate = connect.gate_of(h, ctx)
+        ctx.may_defer = may_defer
+        connect.write(y, gate, x, ctx)
+
+    def forward(self, x: torch.Tensor, ctx: StepContext, unit: CacheUnitView, writes_cache: bool) -> None:
+        self._sublayer(self.connect1, lambda h, y: self.mixer.compute(h, y, ctx, unit, writes_cache), x, ctx)
+        if self.feed_forward is not None:
+            self._sublayer(self.connect2, lambda h, y: self.feed_forward.compute(h, y, ctx), x, ctx)

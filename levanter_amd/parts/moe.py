@@ -11,6 +11,11 @@ Nothing of the routing goes to the host: a kernel orders the step's (token, choi
 stretch into row tiles, and the two products run over the tiles with a grid sized for the worst case (workgroups beyond the
 tiles that exist return at once), so the launches depend on the number of tokens alone and a step can be replayed from a
 HIP graph. Experts whose inner width is no multiple of 8 carry zeros behind it.
+
+Switches beside that: ``score`` "softmax" (the scores are the softmax of z over all router outputs); ``n_identity`` router outputs
+behind the experts' that stand for experts without weights whose result is their input (they take part in scores, groups and
+choice like any other); ``limit`` and ``up_shift`` in the experts' activation, act(min(gate, limit)) * (clamp(up, +-limit) +
+up_shift); ``shared``, the description of a feed-forward that runs for every token and is added.
 """
 from __future__ import annotations
 
@@ -21,15 +26,17 @@ import torch
 from levanter_amd.kernels.library import ACTIVATIONS
 from .base import BuildEnv, FeedForward, StepContext
 from .linear import Linear
-from .registry import FEED_FORWARDS
+from .embedding import tensors_of_nested
+from .registry import FEED_FORWARDS, part_class
 from .spec import PartSpec
 
 
 @FEED_FORWARDS.register("routed_experts")
 class RoutedExperts(FeedForward):
     """params: ``dim``, ``inner_dim``, ``n_experts``, ``top``, ``n_groups`` (1), ``keep`` (1), ``group_top`` (2), ``activation``
-    ("silu"), ``renormalize`` (False), ``correction`` (True: the tensor exists). Tensors: ``router.weight`` ``[E, dim]``,
-    ``correction`` ``[E]``, and per expert e ``experts.<e>.gate.weight``, ``experts.<e>.up.weight`` ``[inner, dim]``,
+    ("silu"), ``renormalize`` (False), ``correction`` (True: the tensor exists), ``score`` ("sigmoid" or "softmax"), ``n_identity`` (0),
+    ``limit`` (None), ``up_shift`` (0), ``shared`` (None, or the description of a feed-forward). Tensors: ``router.weight`` ``[E + n_identity, dim]``,
+    ``correction`` ``[E + n_identity]``, and per expert e ``experts.<e>.gate.weight``, ``experts.<e>.up.weight`` ``[inner, dim]``,
     ``experts.<e>.down.weight`` ``[dim, inner]``."""
 
     graph_safe = True
@@ -44,8 +51,15 @@ class RoutedExperts(FeedForward):
         if self.activation not in ACTIVATIONS:
             raise ValueError(f"routed_experts: unknown activation {self.activation!r}")
         E, D, F = self.n_experts, self.dim, self.inner
-        if E % self.n_groups or not 0 < self.keep <= self.n_groups or not 0 < self.top <= self.keep * (E // self.n_groups):
-            raise ValueError(f"routed_experts: {E} experts in {self.n_groups} groups, {self.keep} kept, {self.top} used")
+        self.n_identity = int(p.get("n_identity", 0))
+        N = self.n_outputs = E + self.n_identity  # what the router chooses among
+        self.score = p.get("score", "sigmoid")
+        if self.score not in ("sigmoid", "softmax"):
+            raise ValueError(f"routed_experts: the scores are 'sigmoid' or 'softmax', got {self.score!r}")
+        self.limit = float(p["limit"]) if p.get("limit") else 0.0
+        self.up_shift = float(p.get("up_shift", 0.0))
+        if N % self.n_groups or not 0 < self.keep <= self.n_groups or not 0 < self.top <= self.keep * (N // self.n_groups):
+            raise ValueError(f"routed_experts: {N} experts in {self.n_groups} groups, {self.keep} kept, {self.top} used")
         Fp = self.inner_padded = (F + 7) // 8 * 8
 
         def f32(name, shape):
@@ -54,8 +68,13 @@ class RoutedExperts(FeedForward):
                 raise ValueError(f"routed_experts: {name} must be {list(shape)}, got {list(t.shape)}")
             return t
 
-        self.router = Linear(f32("router.weight", (E, D)), None, "out_in", env)
-        self.correction = f32("correction", (E,)).to(env.device).contiguous() if p.get("correction", True) else None
+        self.router = Linear(f32("router.weight", (N, D)), None, "out_in", env)
+        self.correction = f32("correction", (N,)).to(env.device).contiguous() if p.get("correction", True) else None
+        shared: PartSpec = p.get("shared")
+        self.shared = None
+        if shared is not None:
+            self.shared = part_class(shared.kind, shared.family or "feed_forward")(shared, tensors_of_nested("shared", tensors), env)
+            self.graph_safe = bool(self.shared.graph_safe)
         # [E, gate rows then up rows, dim] and [E, dim, inner]
         w_in = torch.zeros(E, 2 * Fp, D)
         w_down = torch.zeros(E, D, Fp)
@@ -79,7 +98,7 @@ class RoutedExperts(FeedForward):
 
     def _run(self, h: torch.Tensor, y: torch.Tensor, ctx: StepContext, accumulate: bool, z=None) -> None:
         K = ctx.kernels
-        T, E, top = h.shape[0], self.n_experts, self.top
+        T, E, top = h.shape[0], self.n_outputs, self.top
         dev = h.device
         if z is None:
             z = self.router(h, ctx, out_dtype=torch.float32)
@@ -87,14 +106,24 @@ class RoutedExperts(FeedForward):
             ctx.settle()  # the sum below reads the residual stream itself
         chosen = torch.empty((T, top), dtype=torch.int32, device=dev)
         weights = torch.empty((T, top), dtype=torch.float32, device=dev)
-        K.moe_route(z, self.correction, chosen, weights, n_groups=self.n_groups, keep=self.keep, group_top=self.group_top, renormalize=self.renormalize)
+        more = {"softmax": True} if self.score == "softmax" else {}
+        K.moe_route(z, self.correction, chosen, weights, n_groups=self.n_groups, keep=self.keep, group_top=self.group_top, renormalize=self.renormalize, **more)
         P = T * top
         rows = K.moe_tile_rows(P, E)  # prompts: four row tiles on every weight fragment a wave loads
         tables = torch.empty(2 * P + 3 * K.moe_max_tiles(P, E, rows) + 1, dtype=torch.int32, device=dev)
         sorted_pairs, pos_of, meta, tiles = tables[:P], tables[P:2 * P], tables[2 * P:2 * P + 1], tables[2 * P + 1:]
-        K.moe_sort(chosen, E, sorted_pairs, pos_of, tiles, meta, tile_rows=rows)
+        own = {"n_real": self.n_experts} if self.n_identity else {}
+        K.moe_sort(chosen, E, sorted_pairs, pos_of, tiles, meta, tile_rows=rows, **own)
         inner = ctx.empty(P, self.inner_padded)
-        K.moe_linear(h, self.w_in, inner, tiles, meta, sorted_pairs, top=top, gather=True, glu=True, activation=self.activation, tile_rows=rows)
+        clamp = {"limit": self.limit, "up_shift": self.up_shift} if self.limit or self.up_shift else {}
+        K.moe_linear(h, self.w_in, inner, tiles, meta, sorted_pairs, top=top, gather=True, glu=True, activation=self.activation, tile_rows=rows, **clamp)
         expert_out = ctx.empty(P, self.dim, torch.float32)
         K.moe_linear(inner, self.w_down, expert_out, tiles, meta, sorted_pairs, top=top, gather=False, tile_rows=rows)
-        K.moe_combine(expert_out, pos_of, weights, y, accumulate=accumulate)
+        if self.n_identity:
+            K.moe_combine(expert_out, pos_of, weights, y, accumulate=accumulate, chosen=chosen, n_real=self.n_experts, identity_in=h)
+        else:
+            K.moe_combine(expert_out, pos_of, weights, y, accumulate=accumulate)
+        if self.shared is not None:
+            may_defer, ctx.may_defer = ctx.may_defer, False  # y is not the residual stream: its sum is finished here
+            self.shared.forward(h, y, ctx)  # added to the experts' sum
+            ctx.may_defer = may_defer

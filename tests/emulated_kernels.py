@@ -78,6 +78,20 @@ class EmulatedKernels:
             x = x + pos_table[positions.long()].float()
         out.copy_(x * scale)
 
+    def pair_embed_add(self, tokens, positions, token_slots, last_token, table, x, buckets, mul_prev, mul_cur) -> None:
+        T = x.shape[0]
+        before = last_token.clone()
+        for t in range(T):
+            slot, pos = int(token_slots[t]), int(positions[t])
+            row = buckets
+            if slot >= 0 and pos > 0:
+                inside = t > 0 and int(token_slots[t - 1]) == slot and int(positions[t - 1]) == pos - 1
+                prev = int(tokens[t - 1]) if inside else int(before[slot])
+                row = (prev * mul_prev + int(tokens[t]) * mul_cur) % buckets
+            x[t] += table[row].float()
+            if slot >= 0 and (t + 1 >= T or int(token_slots[t + 1]) != slot):
+                last_token[slot] = int(tokens[t])
+
     def feed_tokens(self, dst, src, rows, n) -> None:
         dst[:n] = src[:n] if rows is None else src[rows[:n].long()]
 
@@ -122,10 +136,10 @@ class EmulatedKernels:
         return None
 
     # ---- rotation of pairs
-    def rotary_pairs(self, q, k, head_dim, freqs, positions) -> None:
+    def rotary_pairs(self, q, k, head_dim, freqs, positions, magnitude=1.0) -> None:
         n = 2 * freqs.numel()
         a = positions.float()[:, None] * freqs[None, :]
-        cos, sin = torch.cos(a)[:, None, :], torch.sin(a)[:, None, :]
+        cos, sin = (torch.cos(a) * magnitude)[:, None, :], (torch.sin(a) * magnitude)[:, None, :]
         for t in (q, k):
             if t is None:
                 continue
@@ -198,7 +212,7 @@ class EmulatedKernels:
         return (parts / torch.sqrt((parts * parts).mean(-1, keepdim=True) + eps)).reshape(T, D) * w
 
     def group_norm_step(self, x, *, groups, eps, y=None, gate=None, post_weight=None, mult=1.0, weight=None, h_out=None, rows=None, defer=False,
-                        pending=None):
+                        pending=None, plain_read=False):
         if pending is not None:
             assert pending.out is x and y is None
             y, gate, post_weight, mult = pending.y, pending.gate, pending.post_weight, pending.mult
@@ -214,7 +228,7 @@ class EmulatedKernels:
                 x.copy_(cur)
         if h_out is not None:
             src = cur if rows is None else cur[rows.long()]
-            h_out.copy_(self._group_norm(src, weight, groups, eps).to(h_out.dtype))
+            h_out.copy_((src if plain_read else self._group_norm(src, weight, groups, eps)).to(h_out.dtype))
         return None
 
     # ---- rotation, rotate-half layout
@@ -250,11 +264,45 @@ class EmulatedKernels:
             o = o / torch.sqrt((o * o).mean(-1, keepdim=True) + norm_eps) * nw * torch.sigmoid(g[t].float().view(H, d))
             out[t] = o.reshape(-1).to(out.dtype)
 
+    # ---- gated linear attention
+    def gated_linear_attention(self, q, k, v, g, z, norm_weight, state, token_slots, out, n_heads, key_dim, value_dim, tau, q_scale, norm_eps,
+                               gate="silu", max_runs=None) -> None:
+        T, H, dk, dv = q.shape[0], n_heads, key_dim, value_dim
+        nw = norm_weight.view(H, dv)
+        for t in range(T):
+            slot = int(token_slots[t])
+            if slot < 0:
+                out[t] = 0
+                continue
+            qf, kf = (u[t].float().view(H, dk) for u in (q, k))
+            vf, gf = (u[t].float().view(H, dv) for u in (v, g))
+            a = torch.exp(-F.softplus(-z[t].float().view(H, dk)) / tau)
+            S = a[:, :, None] * state[slot] + kf[:, :, None] * vf[:, None, :]
+            state[slot] = S
+            o = torch.einsum("hij,hi->hj", S, qf * q_scale)
+            o = o / torch.sqrt((o * o).mean(-1, keepdim=True) + norm_eps) * nw
+            o = o * (gf * torch.sigmoid(gf) if gate == "silu" else torch.sigmoid(gf))
+            out[t] = o.reshape(-1).to(out.dtype)
+
+    # ---- row kernels of gated feed-forwards and of branches with norms of their own
+    def glu_activate(self, z, out, activation, limit=0.0, up_shift=0.0) -> None:
+        F_ = z.shape[1] // 2
+        gt, up = z[:, :F_].float(), z[:, F_:].float()
+        if limit > 0:
+            gt, up = gt.clamp(max=limit), up.clamp(-limit, limit)
+        out.copy_((_act(activation)(gt) * (up + up_shift)).to(out.dtype))
+
+    def norm_sum2(self, a, b, weight_a, weight_b, scale_a, scale_b, eps, y) -> None:
+        def n(v, w):
+            return v / torch.sqrt((v * v).mean(-1, keepdim=True) + eps) * w
+
+        y.copy_(scale_a * n(a, weight_a) + scale_b * n(b, weight_b))
+
     # ---- mixture of experts
-    def moe_route(self, z, correction, chosen, weights, *, n_groups=1, keep=1, group_top=2, renormalize=False) -> None:
+    def moe_route(self, z, correction, chosen, weights, *, n_groups=1, keep=1, group_top=2, renormalize=False, softmax=False) -> None:
         T, E = z.shape
         top = chosen.shape[1]
-        s = torch.sigmoid(z.float())
+        s = torch.softmax(z.float(), -1) if softmax else torch.sigmoid(z.float())
         c = s if correction is None else s + correction
         per = E // n_groups
         for t in range(T):
@@ -276,7 +324,7 @@ class EmulatedKernels:
     def moe_max_tiles(self, pairs, n_experts, tile_rows=16) -> int:
         return pairs // tile_rows + n_experts + 1
 
-    def moe_sort(self, chosen, n_experts, sorted_pairs, pos_of, tiles, meta, tile_rows=16) -> None:
+    def moe_sort(self, chosen, n_experts, sorted_pairs, pos_of, tiles, meta, tile_rows=16, n_real=None) -> None:
         flat = chosen.reshape(-1).long()
         order = torch.sort(flat, stable=True).indices
         P = flat.numel()
@@ -286,13 +334,13 @@ class EmulatedKernels:
         n, at = 0, 0
         for e in range(n_experts):
             count = int((flat == e).sum())
-            for i in range(0, count, tile_rows):
+            for i in range(0, count if n_real is None or e < n_real else 0, tile_rows):
                 tl[n] = torch.tensor([e, at + i, min(tile_rows, count - i)], dtype=torch.int32)
                 n += 1
             at += count
         meta[0] = n
 
-    def moe_linear(self, a, w, out, tiles, meta, sorted_pairs, *, top, gather, glu=False, activation="none", tile_rows=16) -> None:
+    def moe_linear(self, a, w, out, tiles, meta, sorted_pairs, *, top, gather, glu=False, activation="none", tile_rows=16, limit=0.0, up_shift=0.0) -> None:
         tl = tiles.view(-1, 3)
         F_ = out.shape[1]
         for i in range(int(meta[0])):
@@ -301,14 +349,20 @@ class EmulatedKernels:
             src = (sorted_pairs[pos].long() // top) if gather else pos
             y = a[src].float() @ w[e].float().t()
             if glu:
-                y = _act(activation)(y[:, :F_]) * y[:, F_:]
+                gt, up = y[:, :F_], y[:, F_:]
+                if limit > 0:
+                    gt, up = gt.clamp(max=limit), up.clamp(-limit, limit)
+                y = _act(activation)(gt) * (up + up_shift)
             out[pos] = y.to(out.dtype)
 
-    def moe_combine(self, expert_out, pos_of, weights, y, accumulate=False) -> None:
+    def moe_combine(self, expert_out, pos_of, weights, y, accumulate=False, chosen=None, n_real=0, identity_in=None) -> None:
         T, top = weights.shape
         acc = y.clone() if accumulate else torch.zeros_like(y)
         for c in range(top):
-            acc = acc + weights[:, c:c + 1] * expert_out[pos_of.view(T, top)[:, c].long()]
+            term = expert_out[pos_of.view(T, top)[:, c].long()]
+            if identity_in is not None:
+                term = torch.where((chosen[:, c] >= n_real)[:, None], identity_in.float(), term)
+            acc = acc + weights[:, c:c + 1] * term
         y.copy_(acc)
 
     # ---- linear
@@ -347,7 +401,7 @@ class EmulatedKernels:
         kv_ = self.k_view(k_pages, n_kv_heads, head_dim, page_size)
         vv_ = self.v_view(v_pages, n_kv_heads, head_dim if value_dim is None else value_dim, page_size)
         ks, vs = [], []
-        for p in range(lo, hi):
+        for p in (lo if hi is None else range(lo, hi)):  # lo may be a list of positions
             page = int(table_row[p // page_size])
             assert page >= 0, "a key inside the window has no page"
             ks.append(kv_[page, :, :, p % page_size, :].reshape(n_kv_heads, head_dim))
@@ -396,13 +450,17 @@ class EmulatedKernels:
             v.copy_(((1.0 - lam) * v.float() + lam * v_first.float()).to(v.dtype))
 
     def head_prepare_write(self, q, k, v, k_pages, v_pages, dest, n_heads, n_kv_heads, head_dim, value_dim, page_size, eps, v_first=None,
-                           blend=None, norm_dim=None, rotary_freqs=None, positions=None) -> None:
+                           blend=None, norm_dim=None, rotary_freqs=None, positions=None, q_norm_weight=None, k_norm_weight=None,
+                           rotary_magnitude=1.0) -> None:
         k, v = k.clone(), v.clone()
-        if rotary_freqs is not None:
-            self.rotary_pairs(q, k, head_dim, rotary_freqs, positions)
+        weighted = q_norm_weight is not None or k_norm_weight is not None
+        if rotary_freqs is not None and not weighted:
+            self.rotary_pairs(q, k, head_dim, rotary_freqs, positions, rotary_magnitude)
         if eps is not None:
-            self.head_prepare(q, n_heads, head_dim, eps, norm_dim=norm_dim)
-            self.head_prepare(k, n_kv_heads, head_dim, eps, norm_dim=norm_dim)
+            self.head_prepare(q, n_heads, head_dim, eps, norm_dim=norm_dim, norm_weight=q_norm_weight)
+            self.head_prepare(k, n_kv_heads, head_dim, eps, norm_dim=norm_dim, norm_weight=k_norm_weight)
+        if rotary_freqs is not None and weighted:  # a norm with a weight comes before the rotation
+            self.rotary_pairs(q, k, head_dim, rotary_freqs, positions, rotary_magnitude)
         if v_first is not None:
             self.head_prepare(None, 0, 0, 0.0, v=v, v_first=v_first, n_blend=n_kv_heads, value_dim=value_dim, blend=blend)
         self.kv_write(k, v, k_pages, v_pages, dest, n_kv_heads, head_dim, page_size, value_dim=value_dim)
@@ -437,7 +495,7 @@ class EmulatedKernels:
 
         out.copy_((c[0] * n(u) + c[1] * n(u * u) + c[2] * n(u * u * u) + c[3]).to(out.dtype))
 
-    def head_talk(self, o, talk, gate, out, n_heads, n_kv_heads, value_dim, out_scale=1.0) -> None:
+    def head_talk(self, o, talk, gate, out, n_heads, n_kv_heads, value_dim, out_scale=1.0, gate_elements=False) -> None:
         T = out.shape[0]
         if talk is None:
             a = o.view(T, n_heads, value_dim)
@@ -446,7 +504,7 @@ class EmulatedKernels:
             own = torch.arange(n_heads) // (n_heads // n_kv_heads)
             a = torch.einsum("hg,tghd->thd", talk.float(), ov[:, :, own, :])  # [t, g, h, d]: weights of g on the values of h's own head
         if gate is not None:
-            a = a * torch.sigmoid(gate.float())[:, :, None]
+            a = a * (torch.sigmoid(gate.float()).view(T, n_heads, value_dim) if gate_elements else torch.sigmoid(gate.float())[:, :, None])
         out.copy_((a * out_scale).reshape(T, -1).to(out.dtype))
 
     def stream_average(self, streams, x, weights, n, defer=False) -> None:
@@ -457,7 +515,7 @@ class EmulatedKernels:
         x.copy_(acc)
 
     def attention_values(self, q, out, k_pages, v_pages, meta, *, n_heads, n_kv_heads, head_dim, value_dim, all_value_heads, page_size,
-                         scale, window, block_tables, softcap=None, slopes=None, chunk=None, sinks=None) -> None:
+                         scale, window, block_tables, softcap=None, slopes=None, chunk=None, sinks=None, keep_first=0) -> None:
         T = q.shape[0]
         g = n_heads // n_kv_heads
         o = out.view(T, n_heads, n_kv_heads if all_value_heads else 1, value_dim)
@@ -467,12 +525,13 @@ class EmulatedKernels:
             lo = max(0, pos - window + 1) if window else 0
             if chunk:
                 lo = max(lo, pos // chunk * chunk)
-            ks, vs = self.gather_kv(k_pages, v_pages, row, lo, pos + 1, n_kv_heads, head_dim, page_size, value_dim)
+            seen = list(range(min(keep_first, lo))) + list(range(lo, pos + 1))  # the kept first positions, then the window
+            ks, vs = self.gather_kv(k_pages, v_pages, row, seen, None, n_kv_heads, head_dim, page_size, value_dim)
             s = torch.einsum("hd,hnd->hn", q[t].float().view(n_heads, head_dim), ks.float().repeat_interleave(g, 0)) * scale
             if softcap:
                 s = softcap * torch.tanh(s / softcap)
             if slopes is not None:
-                s = s - slopes.float()[:, None] * (pos - torch.arange(lo, pos + 1)).float()[None, :]
+                s = s - slopes.float()[:, None] * (pos - torch.tensor(seen)).float()[None, :]
             if sinks is not None:  # a score without a key and without a value in the denominator
                 p = torch.softmax(torch.cat([s, sinks.float()[:, None]], -1), -1)[:, :-1]
             else:

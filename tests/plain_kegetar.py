@@ -274,3 +274,165 @@ def forward(tokens: List[int], weights: Dict[str, torch.Tensor], cfg: dict) -> T
         streams.append(x.clone())
     hfin = one_plus_norm(x, weights["final.norm"], eps)
     return hfin @ weights["head"].T, streams, margin
+
+
+def plain_logits(W: Dict[str, torch.Tensor], cfg: dict, tokens) -> torch.Tensor:
+    return forward([int(t) for t in tokens], W, cfg)[0]
+
+
+def plain_greedy(W: Dict[str, torch.Tensor], cfg: dict, prompt: List[int], n_new: int) -> List[int]:
+    toks = [int(t) for t in prompt]
+    for _ in range(n_new):
+        toks.append(int(torch.argmax(plain_logits(W, cfg, toks)[-1])))
+    return toks[len(prompt):]
+
+
+# ---- configurations and weights for tests -----------------------------------------------------------------------
+def left_sizes(heads=4, kv_heads=2, dim=16, vdim=8, window=24, keep_first=3, rot_dims=None, base=10000.0, scaling="default", scale=None) -> dict:
+    if scaling == "default":
+        scaling = {"factor": 3.0, "original": 40, "fast": 8.0, "slow": 1.0}
+    rot = None if rot_dims == 0 else {"dims": dim if rot_dims is None else rot_dims, "base": base, **({"scaling": scaling} if scaling else {})}
+    m = {"heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": vdim, "scale": dim ** -0.5 if scale is None else scale}
+    if rot:
+        m["rot"] = rot
+    if window is not None:
+        m["mask"] = {"size": window, "keep_first": keep_first}
+    return m
+
+
+def right_sizes(heads=2, dim=16, vdim=8, tau=8.0, decay_rank=4) -> dict:
+    return {"heads": heads, "dim": dim, "vdim": vdim, "tau": tau, "decay_rank": decay_rank}
+
+
+def parallel_layer(left=None, right=None, mlp="dense", weights_of=None) -> dict:
+    L = {"type": "parallel", "mixer": {"left": left or left_sizes(), "right": right or right_sizes()}, "mlp": dense_mlp() if mlp == "dense" else mlp}
+    if weights_of is not None:
+        L["weights_of"] = weights_of
+    return L
+
+
+def attention_layer(heads=4, kv_heads=1, dim=16, window=20, scale=None, mlp="dense", weights_of=None) -> dict:
+    m = {"heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": dim, "scale": dim ** -0.5 if scale is None else scale}
+    if window is not None:
+        m["mask"] = {"size": window}
+    L = {"type": "attention", "mixer": m, "mlp": dense_mlp() if mlp == "dense" else mlp}
+    if weights_of is not None:
+        L["weights_of"] = weights_of
+    return L
+
+
+def dense_mlp(ff=48) -> dict:
+    return {"kind": "dense", "ff": ff}
+
+
+def experts_mlp(ff=24, experts=6, top=2, identity=2, groups=(2, 1), limit=2.0, shared=32, shared_limit=1.5) -> dict:
+    router = {"experts": experts, "top": top, "identity": identity}
+    if groups:
+        router["groups"] = {"count": groups[0], "keep": groups[1]}
+    mlp = {"kind": "moe", "expert": {"ff": ff, "limit": limit}, "router": router}
+    if shared:
+        mlp["shared"] = {"ff": shared, "limit": shared_limit}
+    return mlp
+
+
+def make_config(vocab=97, width=64, layers=None, eps=1e-5, mult=0.7, bigram=(31, 5, 3)) -> dict:
+    cfg = {"architecture": "Kegetar", "vocab": vocab, "width": width, "norm": {"eps": eps}, "residual_mult": mult,
+           "layers": layers if layers is not None else [parallel_layer(), attention_layer()]}
+    if bigram:
+        cfg["embedding"] = {"bigram": {"buckets": bigram[0], "mul_prev": bigram[1], "mul_cur": bigram[2]}}
+    return cfg
+
+
+def random_weights(cfg: dict, seed: int, dtype=F64, clear_routing: bool = False) -> Dict[str, torch.Tensor]:
+    """Weights drawn so that every mechanism matters: scores of order one, gates that are not saturated, decays over a wide
+    range, activations that reach their limits, router scores whose order the correction changes. Values are bfloat16 numbers
+    (a file stores them exactly). ``clear_routing``: routers that decide by a wide margin (scores that move little with the
+    input, corrections a fixed step apart in a random order), for runs in 16-bit arithmetic, where a choice by less than the
+    inputs' rounding could fall either way."""
+    g = torch.Generator().manual_seed(seed)
+    D, V = cfg["width"], cfg["vocab"]
+
+    def rn(*shape, std=1.0):
+        return (torch.randn(*shape, generator=g) * std).to(torch.bfloat16).to(dtype)
+
+    W = {"embed": rn(V, D), "final.norm": rn(D, std=0.2), "head": rn(V, D, std=1 / math.sqrt(D))}
+    b = (cfg.get("embedding") or {}).get("bigram")
+    if b:
+        W["bigram"] = rn(b["buckets"] + 1, D, std=0.7)
+    lin = 1 / math.sqrt(D)
+    for i, L in enumerate(cfg["layers"]):
+        if L.get("weights_of") is not None:
+            continue
+        m, p = L["mixer"], f"l{i}."
+        W[p + "norm1"] = rn(D, std=0.2)
+        if L["type"] == "parallel":
+            le, ri = m["left"], m["right"]
+            H, G, dk, dv = le["heads"], le["kv_heads"], le["dim"], le["vdim"]
+            q = p + "mix.left."
+            W[q + "q"], W[q + "k"], W[q + "v"] = rn(H * dk, D, std=lin), rn(G * dk, D, std=lin), rn(G * dv, D, std=lin)
+            W[q + "q.norm"], W[q + "k.norm"] = 1.5 + rn(dk, std=0.3), 1.5 + rn(dk, std=0.3)
+            W[q + "g"] = rn(H * dv, D, std=1.5 * lin)
+            W[q + "o"] = rn(D, H * dv, std=1 / math.sqrt(H * dv))
+            W[p + "mix.left.out"] = 1 + rn(D, std=0.2)
+            H, dk, dv, rank = ri["heads"], ri["dim"], ri["vdim"], ri["decay_rank"]
+            q = p + "mix.right."
+            W[q + "q"], W[q + "k"] = rn(H * dk, D, std=lin), rn(H * dk, D, std=lin)
+            W[q + "v"], W[q + "g"] = rn(H * dv, D, std=lin), rn(H * dv, D, std=1.5 * lin)
+            W[q + "a1"] = rn(rank, D, std=lin)
+            W[q + "a2"] = rn(H * dk, rank, std=2 / math.sqrt(rank))
+            W[q + "a2.b"] = rn(H * dk, std=2.0)
+            W[q + "norm"] = 1 + rn(dv, std=0.2)
+            W[q + "o"] = rn(D, H * dv, std=1 / math.sqrt(H * dv))
+            W[p + "mix.right.out"] = 1 + rn(D, std=0.2)
+        else:
+            H, G, dk = m["heads"], m["kv_heads"], m["dim"]
+            q = p + "mix."
+            W[q + "q"], W[q + "q.b"] = rn(H * dk, D, std=lin), rn(H * dk, std=0.3)
+            W[q + "k"], W[q + "k.b"] = rn(G * dk, D, std=lin), rn(G * dk, std=0.3)
+            W[q + "q.norm"], W[q + "k.norm"] = 1.5 + rn(H * dk, std=0.3), 1.5 + rn(G * dk, std=0.3)
+            W[q + "o"] = rn(D, H * dk, std=1 / math.sqrt(H * dk))
+        mlp = L.get("mlp")
+        if mlp is None:
+            continue
+        W[p + "norm2"] = rn(D, std=0.2)
+        q = p + "mlp."
+        if mlp["kind"] == "dense":
+            F = mlp["ff"]
+            W[q + "gate"], W[q + "gate.b"] = rn(F, D, std=lin), rn(F, std=0.3)
+            W[q + "up"], W[q + "up.b"] = rn(F, D, std=lin), rn(F, std=0.3)
+            W[q + "down"], W[q + "down.b"] = rn(D, F, std=1 / math.sqrt(F)), rn(D, std=0.3)
+            continue
+        F, r = mlp["expert"]["ff"], mlp["router"]
+        E, N = r["experts"], r["experts"] + r.get("identity", 0)
+        W[q + "router"] = rn(N, D, std=(0.02 if clear_routing else 1.5) * lin)
+        W[q + "correction"] = rn(N, std=0.1)
+        if clear_routing:
+            W[q + "correction"] = (torch.randperm(N, generator=g).to(torch.float32) * 0.0625 - 0.25).to(torch.bfloat16).to(dtype)
+        for e in range(E):
+            W[q + f"e{e}.gate"], W[q + f"e{e}.up"] = rn(F, D, std=2 * lin), rn(F, D, std=2 * lin)
+            W[q + f"e{e}.down"] = rn(D, F, std=1 / math.sqrt(F))
+        sh = mlp.get("shared")
+        if sh:
+            W[q + "shared.gate"], W[q + "shared.up"] = rn(sh["ff"], D, std=2 * lin), rn(sh["ff"], D, std=2 * lin)
+            W[q + "shared.down"] = rn(D, sh["ff"], std=1 / math.sqrt(sh["ff"]))
+    return W
+
+
+def write_folder(cfg: dict, W: Dict[str, torch.Tensor], path: str, dtype=torch.bfloat16) -> str:
+    """config.json and model.safetensors of these weights, through the safetensors package. The inner size of the decay's map
+    is left to the tensors: the written configuration does not name it."""
+    import copy
+    import json
+    import os
+
+    from safetensors.torch import save_file
+
+    os.makedirs(path, exist_ok=True)
+    out = copy.deepcopy(cfg)
+    for L in out["layers"]:
+        if L["type"] == "parallel":
+            L["mixer"]["right"].pop("decay_rank", None)
+    with open(os.path.join(path, "config.json"), "w") as f:
+        json.dump(out, f)
+    save_file({k: v.to(dtype).contiguous() for k, v in W.items()}, os.path.join(path, "model.safetensors"))
+    return path

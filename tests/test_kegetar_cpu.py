@@ -1,0 +1,359 @@
+"""Kegetar through the framework's step function, cache manager and parts on the CPU with the emulated kernels, against the
+plain implementation: what differs here is a fault of the host logic (tables, pages that a window gives back while the first
+positions stay, state slots, the token before a step's first, layers that run another layer's weights), not of a kernel. Also
+the plain implementation's own mechanisms against direct statements of what they must do."""
+import copy
+import math
+import os
+
+import pytest
+import torch
+
+import plain_kegetar as P
+import traces as TR
+from emulated_kernels import EmulatedKernels
+from kegetar_configs import KEG
+from levanter_amd.cache import PagedKv, SlotState
+from levanter_amd.config import ConfigError, InferenceEngineConfig, KegetarConfig, LmConfig
+from levanter_amd.engine import ModelRunner, StepEntry
+from levanter_amd.engine.loading import load_model, make_cache
+from levanter_amd.parts import BuildEnv
+from levanter_amd.parts.position import rotary_frequencies
+from levanter_amd.weights import WeightsError
+
+
+def build(name, tmp, dtype=torch.float32):
+    raw, seed = KEG[name]
+    W = P.random_weights(raw, seed)
+    d = P.write_folder(raw, W, os.path.join(str(tmp), name), torch.float32)
+    env = BuildEnv(dtype, torch.device("cpu"), EmulatedKernels())
+    config, model = load_model(d, env)
+    return raw, W, model, env, config
+
+
+def close(got: torch.Tensor, want: torch.Tensor) -> None:
+    """Equal to 2e-4, but for one element in a hundred ten times that: a request's first token gives the linear attention's state one
+    outer product, (q . k) v read back; where q . k nearly cancels the head norm divides a number of the size of sqrt(eps) by itself and
+    multiplies the 32-bit sum's last bits by 1 / sqrt(eps)."""
+    torch.testing.assert_close(got, want, rtol=2e-3, atol=2e-3)
+    bad = ((got - want).abs() > 2e-4 + 2e-4 * want.abs()).double().mean()
+    assert float(bad) <= 0.01, f"{float(bad):.3%} of the elements differ by more than 2e-4"
+
+
+LENGTHS = {"A": [70, 45, 100, 37, 64, 33], "B": [90, 130, 41, 17, 64], "C": [40, 12, 90]}
+
+
+@pytest.fixture(scope="module", params=list(KEG))
+def setup(request, tmp_path_factory):
+    raw, W, model, env, _ = build(request.param, tmp_path_factory.mktemp("keg"))
+    reqs = TR.random_requests(raw["vocab"], LENGTHS[request.param], 5)
+    plain = {rid: P.plain_logits(W, raw, t) for rid, t in reqs.items()}
+    return raw, W, model, env, reqs, plain
+
+
+def replay(model, env, steps, max_tokens, ps=16, max_seqs=4, after_step=None):
+    cfg = InferenceEngineConfig(max_pages=max(1, max_tokens // ps), max_seqs=max_seqs, page_size=ps, max_pages_per_seq=16, compute_dtype="float32")
+    cache = make_cache(model, cfg)
+    runner = ModelRunner(model, cache, env)
+    live, out = {}, {}
+    for s in steps:
+        entries = []
+        for e in s["entries"]:
+            if e["id"] not in live:
+                live[e["id"]] = cache.open(e["id"])
+            entries.append(StepEntry(live[e["id"]], e["tokens"], e["want"]))
+        logits = runner.step(entries)
+        cache.check_invariants()
+        if after_step is not None:
+            after_step(cache, live)
+        if logits.shape[0]:
+            out[s["step"]] = logits
+        for rid in s["end"]:
+            cache.close(live.pop(rid))
+    cache.check_invariants()
+    assert all(g.pool.n_free == g.pool.n_pages for g in cache.groups)
+    return out, cache
+
+
+@pytest.mark.parametrize("mode", ["whole", "singles", "portions", "mixed"])
+def test_every_way_of_cutting_gives_the_plain_logits(setup, mode):
+    raw, W, model, env, reqs, plain = setup
+    steps = {"whole": TR.trace_whole, "singles": TR.trace_prefill_then_singles, "portions": TR.trace_portions,
+             "mixed": lambda r: TR.trace_mixed(r, seed=4)}[mode](reqs)
+    TR.number(steps)
+    got, _ = replay(model, env, steps, TR.peak_tokens(steps))
+    want = TR.expected_rows(steps, lambda rid: plain[rid[1:]])
+    assert set(got) == set(want)
+    for k in want:
+        close(got[k].double(), want[k])
+
+
+def test_the_registry_finds_the_architecture_and_a_layer_may_run_anothers_weights(tmp_path):
+    raw, W, model, env, config = build("A", tmp_path)
+    assert isinstance(config, KegetarConfig) and config.model_type_name == "kegetar"
+    assert LmConfig.from_dict(config.to_hf_config()) == config
+    # four layers have tensors; layers 4 and 5 run those of layers 0 and 3, each entry with a cache unit of its own
+    assert [b.kind for b in model.blocks] == ["post_norm"] * 4
+    assert [(e.layer, e.cache, e.writes_cache) for e in model.plan] == [(0, 0, True), (1, 1, True), (2, 2, True), (3, 3, True), (0, 4, True), (3, 5, True)]
+    reqs = dict(model.cache_requirements())
+    left = PagedKv(2, 16, 24, value_dim=8, keep_first=3)
+    assert reqs[0].paged() == reqs[4].paged() == left and reqs[0].slot_state() == SlotState((2, 16, 8), "float32")
+    assert reqs[1].paged() == PagedKv(4, 16, 17, keep_first=5) and reqs[1].slot_state() == SlotState((2, 8, 16), "float32")
+    assert reqs[2] == PagedKv(1, 16, 20) and reqs[3] == reqs[5] == PagedKv(2, 24, 9)
+    assert reqs[-1] == SlotState((1,), "int32")  # the token before a step's first, kept by the embedding
+    # the inner size of the decay's map is what the tensors say: the written configuration does not name it
+    assert "decay_rank" not in config.layers[0]["mixer"]["right"] and model.blocks[0].mixer.branches[1].rank == 4
+    # a window that is absent keeps everything, and then there are no first positions to keep
+    _, _, model_b, _, _ = build("B", tmp_path)
+    assert dict(model_b.cache_requirements())[2].paged() == PagedKv(3, 8, None)
+    assert dict(model_b.cache_requirements()).get(-1) is None  # no pair table: nothing to keep
+
+
+def test_the_residual_stream_after_every_layer(tmp_path):
+    import levanter_amd.parts.gated_block as GB
+
+    raw, W, model, env, _ = build("A", tmp_path)
+    toks = TR.random_requests(raw["vocab"], [29], 3)["r0"]
+    _, want, _ = P.forward(toks, W, raw)
+    got = []
+    orig = GB.PostNormBlock.forward
+
+    def fwd(self, x, ctx, unit, wc):
+        orig(self, x, ctx, unit, wc)
+        assert ctx.pending is not None  # the last sublayer's write waits for the pass that reads the stream next
+        ctx.settle()
+        got.append(x.clone())
+
+    GB.PostNormBlock.forward = fwd
+    try:
+        cache = make_cache(model, InferenceEngineConfig(max_pages=8, max_seqs=2, page_size=16, max_pages_per_seq=8, compute_dtype="float32"))
+        ModelRunner(model, cache, env).step([StepEntry(cache.open("a"), toks, [])])
+    finally:
+        GB.PostNormBlock.forward = orig
+    assert len(got) == len(want) == 6
+    for g, w in zip(got, want):
+        torch.testing.assert_close(g.double(), w, rtol=1e-4, atol=1e-4)
+
+
+def test_windowed_groups_give_pages_back_keep_the_first_positions_and_take_used_ones(tmp_path):
+    """Requests of 130 and 60 tokens in portions: a group with a window never holds more than the window, a portion and the
+    blocks of its kept first positions need; those blocks stay for good; pages freed behind the window are handed out again."""
+    raw, W, model, env, _ = build("B", tmp_path)
+    reqs = TR.random_requests(raw["vocab"], [130, 60], 9)
+    steps = TR.number(TR.trace_portions(reqs, sizes=[7, 2, 13, 3, 5]))
+    seen = {}
+
+    def after(cache, live):
+        for g in cache.groups:
+            r = g.requirement
+            if r.window is None:
+                continue
+            kept = -(-r.keep_first // 16)
+            for rid, h in live.items():
+                held = len(g.pages_held(h.slot))
+                blocks = -(-h.length // 16)
+                first = max(0, h.length - r.window + 1) // 16
+                assert held == blocks - first + min(kept, first)
+                assert all(g.block_tables[h.slot, b] >= 0 for b in range(min(kept, blocks)))
+                seen[(r.window, r.keep_first)] = max(seen.get((r.window, r.keep_first), 0), held)
+
+    got, cache = replay(model, env, steps, 256, after_step=after)
+    assert seen[(5, 9)] <= 3 and seen[(30, 70)] <= 8 and seen[(1, 0)] <= 2
+    plain = {rid: P.plain_logits(W, raw, t) for rid, t in reqs.items()}
+    want = TR.expected_rows(steps, lambda rid: plain[rid[1:]])
+    for k in want:
+        close(got[k].double(), want[k])
+
+
+def test_a_slot_that_is_used_again_starts_from_zero_state_and_without_a_token_before(tmp_path):
+    """Two requests one after the other in an engine of one slot: the second finds the first one's state, last token and pages."""
+    raw, W, model, env, _ = build("A", tmp_path)
+    reqs = TR.random_requests(raw["vocab"], [40, 23], 2)
+    steps = TR.number(TR.trace_prefill_then_singles(reqs, n_single=5))
+    got, _ = replay(model, env, steps, 64, max_seqs=1)
+    plain = {rid: P.plain_logits(W, raw, t) for rid, t in reqs.items()}
+    want = TR.expected_rows(steps, lambda rid: plain[rid[1:]])
+    for k in want:
+        close(got[k].double(), want[k])
+
+
+def test_bad_configurations_and_checkpoints_are_refused(tmp_path):
+    raw, _ = KEG["A"]
+
+    def broken(change):
+        c = copy.deepcopy(raw)
+        change(c)
+        return c
+
+    cases = [
+        lambda c: c["layers"][0].update(type="latent"),
+        lambda c: c["layers"][0]["mixer"].pop("right"),
+        lambda c: c["layers"][0]["mixer"]["left"].update(kv_heads=3),
+        lambda c: c["layers"][0]["mixer"]["left"]["rot"].update(dims=7),
+        lambda c: c["layers"][0]["mixer"]["left"]["rot"].update(dims=18),
+        lambda c: c["layers"][0]["mixer"]["left"]["rot"]["scaling"].pop("slow"),
+        lambda c: c["layers"][0]["mixer"]["left"]["mask"].update(size=0),
+        lambda c: c["layers"][0]["mixer"]["left"]["mask"].update(keep_first=-1),
+        lambda c: c["layers"][0]["mixer"]["right"].update(tau=0),
+        lambda c: c["layers"][2]["mixer"].update(vdim=8),  # the keys are the values
+        lambda c: c["layers"][2]["mixer"]["mask"].update(keep_first=2),  # only the other attention keeps first positions
+        lambda c: c["layers"][2]["mixer"].update(rot={"dims": 8, "base": 100.0}),
+        lambda c: c["layers"][1]["mlp"].update(kind="sparse"),
+        lambda c: c["layers"][1]["mlp"]["expert"].pop("limit"),
+        lambda c: c["layers"][1]["mlp"]["router"].update(top=5),  # more than the kept groups hold
+        lambda c: c["layers"][1]["mlp"]["router"]["groups"].update(count=3),  # 8 router outputs do not split into 3
+        lambda c: c["layers"][4].update(weights_of=4),  # itself
+        lambda c: c["layers"][4].update(weights_of=5),  # a later layer
+        lambda c: c["layers"][5].update(weights_of=4),  # a layer without tensors of its own
+        lambda c: c["layers"][4].update(weights_of=1),  # another description
+        lambda c: c["embedding"]["bigram"].update(buckets=0),
+        lambda c: c.pop("norm"),
+        lambda c: c.pop("width"),
+    ]
+    for i, change in enumerate(cases):
+        with pytest.raises(ConfigError):
+            LmConfig.from_dict(broken(change))
+            pytest.fail(f"case {i} was accepted")
+    # a checkpoint that lacks a tensor, has one too many (tensors of a layer that runs another's) and one of the wrong shape
+    W = P.random_weights(raw, 1)
+    W2 = dict(W)
+    del W2["l0.mix.right.a2.b"]
+    W2["l4.norm1"] = torch.zeros(64, dtype=torch.float64)
+    W2["l1.mlp.correction"] = torch.zeros(6, dtype=torch.float64)  # the identity outputs have entries too
+    d = P.write_folder(raw, W2, str(tmp_path / "bad"), torch.float32)
+    env = BuildEnv(torch.float32, torch.device("cpu"), EmulatedKernels())
+    with pytest.raises(WeightsError) as e:
+        load_model(d, env)
+    assert e.value.missing == ["l0.mix.right.a2.b"] and e.value.unexpected == ["l4.norm1"] and len(e.value.wrong_shape) == 1
+    # the two matrices of the decay's map must agree on their inner size
+    W3 = dict(W)
+    W3["l0.mix.right.a1"] = torch.zeros(7, 64, dtype=torch.float64)
+    d = P.write_folder(raw, W3, str(tmp_path / "bad2"), torch.float32)
+    with pytest.raises(ValueError):
+        load_model(d, env)
+
+
+# ---- the plain implementation's mechanisms against direct statements ------------------------------------------------------
+def test_the_pair_rows():
+    assert P.bigram_rows([4, 9, 0, 9], 11, 3, 5) == [11, (4 * 3 + 9 * 5) % 11, (9 * 3) % 11, (9 * 5) % 11]
+    assert P.bigram_rows([7], 5, 1, 1) == [5]
+
+
+def test_rotation_of_pairs_and_its_magnitude():
+    v = torch.zeros(1, 1, 8, dtype=torch.float64)
+    v[0, 0, 2] = 1.0  # dimension 2 is paired with dimension 3; dimensions 6 and 7 never turn
+    v[0, 0, 7] = 2.0
+    freqs, mag = P.yarn_frequencies(6, 100.0, None)
+    assert mag == 1.0 and freqs == [1.0, 100.0 ** (-2 / 6), 100.0 ** (-4 / 6)]
+    out = P.rotate_pairs(v, torch.tensor([3]), freqs, 1.25)
+    a = 3 * freqs[1]
+    want = torch.zeros(8, dtype=torch.float64)
+    want[2], want[3], want[7] = 1.25 * math.cos(a), 1.25 * math.sin(a), 2.0
+    torch.testing.assert_close(out[0, 0], want)
+    q, k = torch.randn(2, 1, 1, 8, dtype=torch.float64)  # scores depend on the distance alone
+    s = [float((P.rotate_pairs(q, torch.tensor([p + 5]), freqs, 1.0) * P.rotate_pairs(k, torch.tensor([p]), freqs, 1.0)).sum()) for p in (0, 7, 300)]
+    assert abs(s[0] - s[1]) < 1e-9 and abs(s[0] - s[2]) < 1e-9
+
+
+def test_stretched_frequencies_by_hand_and_in_the_package():
+    """8 pairs, base 10000, original length 32: index(t) = 16 ln(32 / (2 pi t)) / (2 ln 10000). fast = 4 gives 0.21 (lo = 0), slow = 1 gives
+    1.41 (hi = 2): pair 0 keeps its frequency, pair 1 is half way, pairs from 2 on turn `factor` times slower."""
+    sc = {"factor": 4.0, "original": 32, "fast": 4.0, "slow": 1.0}
+    freqs, mag = P.yarn_frequencies(16, 10000.0, sc)
+    base = [10000.0 ** (-2 * i / 16) for i in range(8)]
+    assert freqs[0] == base[0] and abs(freqs[1] - (0.5 * base[1] / 4 + 0.5 * base[1])) < 1e-15
+    assert all(abs(f - b / 4) < 1e-15 for f, b in zip(freqs[2:], base[2:]))
+    assert abs(mag - (0.1 * math.log(4.0) + 1.0)) < 1e-15
+    assert rotary_frequencies(16, 10000.0, sc) == freqs  # the package's table, computed on its own
+    # a ramp of no width: everything from lo on is stretched
+    sc = {"factor": 2.0, "original": 32, "fast": 1.0, "slow": 1.0}
+    lo = math.floor(16 * math.log(32 / (2 * math.pi)) / (2 * math.log(10000.0)))
+    freqs, _ = P.yarn_frequencies(16, 10000.0, sc)
+    assert lo == 1 and freqs[0] == base[0] and freqs[1] == base[1] and abs(freqs[2] - base[2] / 2) < 1e-15  # hi = ceil(1.41) = 2
+    assert rotary_frequencies(16, 10000.0, sc) == freqs
+
+
+def test_visibility_as_a_table():
+    ok = P.visible(8, 3, 2)
+    assert ok.tolist() == [[j <= i and (i - j < 3 or j < 2) for j in range(8)] for i in range(8)]
+    assert ok[7].tolist() == [True, True, False, False, False, True, True, True]
+    assert P.visible(5, None, 4).tolist() == [[j <= i for j in range(5)] for i in range(5)]
+    assert P.visible(4, 1).tolist() == [[i == j for j in range(4)] for i in range(4)]
+
+
+def test_the_distance_term():
+    assert P.distance_slopes(4) == [0.25, 0.0625, 0.015625, 0.00390625]
+    # one head, equal keys: the weights fall by exp(-slope) a position
+    q = torch.zeros(3, 1, 2, dtype=torch.float64)
+    k = torch.zeros(3, 1, 2, dtype=torch.float64)
+    v = torch.eye(3, dtype=torch.float64).view(3, 1, 3)
+    o = P.softmax_attention(q, k, v, 1.0, P.visible(3, None), [0.5])
+    w = torch.tensor([math.exp(-1.0), math.exp(-0.5), 1.0], dtype=torch.float64)
+    torch.testing.assert_close(o[2, 0], w / w.sum())
+
+
+def test_gated_linear_attention_by_hand():
+    """One head, two key channels, one value channel, two tokens, written out; and a carried state equals one run."""
+    D = 3
+    W = {"m.q": torch.tensor([[1.0, 0, 0], [0, 1.0, 0]]), "m.k": torch.tensor([[0, 1.0, 0], [1.0, 0, 0]]), "m.v": torch.tensor([[0, 0, 1.0]]),
+         "m.g": torch.tensor([[1.0, 1.0, 0]]), "m.a1": torch.tensor([[1.0, 0, 0]]), "m.a2": torch.tensor([[2.0], [-1.0]]), "m.a2.b": torch.tensor([0.5, 0.0]),
+         "m.norm": torch.tensor([1.0]), "m.o": torch.tensor([[1.0], [0.0], [0.0]])}
+    W = {k: v.double() for k, v in W.items()}
+    m = {"heads": 1, "dim": 2, "vdim": 1, "tau": 2.0}
+    h = torch.tensor([[1.0, 2.0, 3.0], [0.5, -1.0, 2.0]], dtype=torch.float64)
+    out, S = P.gated_linear_attention(h, W, "m", m, 0.0)
+    sig = lambda x: 1 / (1 + math.exp(-x))
+    a1 = [sig(2 * 1.0 + 0.5) ** 0.5, sig(-1.0) ** 0.5]
+    a2 = [sig(2 * 0.5 + 0.5) ** 0.5, sig(-0.5) ** 0.5]
+    S1 = [2.0 * 3.0, 1.0 * 3.0]  # k = (h[1], h[0]), v = h[2]; from zero the decay has nothing to act on
+    S2 = [a2[0] * S1[0] + (-1.0) * 2.0, a2[1] * S1[1] + 0.5 * 2.0]
+    torch.testing.assert_close(S[0, :, 0], torch.tensor(S2, dtype=torch.float64))
+    o2 = (0.5 * S2[0] + (-1.0) * S2[1]) / math.sqrt(2)  # q = (h[0], h[1]) / sqrt(2)
+    g2 = 0.5 - 1.0
+    want = o2 / abs(o2) * g2 * sig(g2)  # the norm of a single channel leaves its sign
+    assert abs(float(out[1, 0]) - want) < 1e-12 and a1[0] > 0
+    first, Sa = P.gated_linear_attention(h[:1], W, "m", m, 0.0)
+    second, Sb = P.gated_linear_attention(h[1:], W, "m", m, 0.0, Sa)
+    torch.testing.assert_close(torch.cat([first, second]), out)
+    torch.testing.assert_close(Sb, S)
+
+
+def test_the_router_by_hand():
+    """Six router outputs in three groups of two, two groups kept, two used; the scores are a softmax over all six; the correction
+    changes the choice, not the weights; a group is scored by its best member; an excluded output counts as minus infinity."""
+    s = [0.3, 0.05, 0.2, 0.15, 0.25, 0.05]
+    z = torch.tensor([[math.log(x) + 1.7 for x in s]], dtype=torch.float64)  # any shift of the logits leaves the softmax
+    none = torch.zeros(6, dtype=torch.float64)
+    chosen, weights, _ = P.route(z, none, 2, 3, 2)
+    assert chosen.tolist() == [[0, 4]]  # groups 0 (0.3) and 2 (0.25) are kept
+    torch.testing.assert_close(weights, torch.tensor([[0.3, 0.25]], dtype=torch.float64))
+    corr = torch.tensor([-0.2, 0.0, 0.0, 0.12, 0.0, 0.0], dtype=torch.float64)
+    chosen, weights, margin = P.route(z, corr, 2, 3, 2)
+    # choice scores 0.1 0.05 | 0.2 0.27 | 0.25 0.05: groups 1 and 2 beat group 0; winners 3 and 4, weights without the correction
+    assert chosen.tolist() == [[3, 4]]
+    torch.testing.assert_close(weights, torch.tensor([[0.15, 0.25]], dtype=torch.float64))
+    assert abs(float(margin[0]) - 0.05) < 1e-12  # between output 4 (0.25) and the best loser, output 2 (0.2)
+    corr = torch.tensor([-1.0, -2.0, -2.0, -2.0, -2.0, -1.5], dtype=torch.float64)
+    # all choice scores negative (-0.7 -1.95 | -1.8 -1.85 | -1.75 -1.45): groups 0 and 2 are kept; three winners from them although output 2 of
+    # the excluded group beats output 1
+    chosen, _, _ = P.route(z, corr, 3, 3, 2)
+    assert chosen.tolist() == [[0, 5, 4]]
+    chosen, _, _ = P.route(z, none, 3, 1, 1)  # one group: the plain top three
+    assert chosen.tolist() == [[0, 4, 2]]
+
+
+def test_experts_that_return_their_input_and_the_clamped_activation():
+    D = 4
+    g = torch.Generator().manual_seed(0)
+    W = {"f.router": torch.zeros(3, D), "f.correction": torch.tensor([0.0, 1.0, 2.0]), "f.e0.gate": torch.randn(5, D, generator=g),
+         "f.e0.up": torch.randn(5, D, generator=g), "f.e0.down": torch.randn(D, 5, generator=g)}
+    W = {k: v.double() for k, v in W.items()}
+    mlp = {"kind": "moe", "expert": {"ff": 5, "limit": 0.7}, "router": {"experts": 1, "top": 2, "identity": 2}}
+    h = torch.randn(6, D, generator=g).double() * 3
+    y, _ = P.expert_feed_forward(h, W, "f", mlp)
+    torch.testing.assert_close(y, 2 * h / 3)  # outputs 1 and 2 win by their corrections: two experts that return h, each with the score 1/3
+    mlp["router"]["top"] = 3
+    y3, _ = P.expert_feed_forward(h, W, "f", mlp)
+    gate, up = (h @ W["f.e0.gate"].T).clamp(max=0.7), (h @ W["f.e0.up"].T).clamp(-0.7, 0.7)
+    assert float((h @ W["f.e0.gate"].T).max()) > 0.7 and float((h @ W["f.e0.up"].T).min()) < -0.7
+    torch.testing.assert_close(y3 - y, ((gate * torch.sigmoid(1.702 * gate) * (up + 1)) @ W["f.e0.down"].T) / 3)

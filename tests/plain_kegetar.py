@@ -404,7 +404,7 @@ def random_weights(cfg: dict, seed: int, dtype=F64, clear_routing: bool = False)
             continue
         F, r = mlp["expert"]["ff"], mlp["router"]
         E, N = r["experts"], r["experts"] + r.get("identity", 0)
-        W[q + "router"] = rn(N, D, std=(0.02 if clear_routing else 1.5) * lin)
+        W[q + "router"] = rn(N, D, std=(0.002 if clear_routing else 0.15) * lin)  # the router reads the stream itself, whose entries are of order ten
         W[q + "correction"] = rn(N, std=0.1)
         if clear_routing:
             W[q + "correction"] = (torch.randperm(N, generator=g).to(torch.float32) * 0.0625 - 0.25).to(torch.bfloat16).to(dtype)
@@ -436,3 +436,10 @@ def write_folder(cfg: dict, W: Dict[str, torch.Tensor], path: str, dtype=torch.b
         json.dump(out, f)
     save_file({k: v.to(dtype).contiguous() for k, v in W.items()}, os.path.join(path, "model.safetensors"))
     return path
+
+
+def first_close_call(W: Dict[str, torch.Tensor], cfg: dict, tokens, delta: float) -> int:
+    """The first position at which some router decides by less than ``delta`` (the number of tokens if there is none)."""
+    margin = forward([int(t) for t in tokens], W, cfg)[2]
+    close = (margin < delta).nonzero()
+    return int(close[0]) if close.numel() else len(tokens)

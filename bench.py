@@ -55,16 +55,18 @@ def main() -> int:
     ap.add_argument("--shape", default="7b", choices=["7b", "xl", "20b"],
                     help="layer sizes of the decode workload: 7b is the headline's; xl and 20b measure the same step at the other "
                          "sizes of the reference's configurations (use --no-points: the prefill point is 2,048 tokens)")
-    ap.add_argument("--workload", default="decode", choices=["decode", "xl_mix", "20b", "zederax", "nakurax", "tativik"],
+    ap.add_argument("--workload", default="decode", choices=["decode", "xl_mix", "20b", "zederax", "nakurax", "tativik", "kegetar"],
                     help="decode: the workload described above. xl_mix / 20b: continuous-batching workloads at the gpt2_xl and gpt2_20b sizes "
                          "through InferenceEngine.generate; they print their own line. zederax: prefill and decode rates of Zederax "
                          "layers at a few sizes beside GPT-2 layers of the same width, heads and inner width; its own line. nakurax: the same for "
                          "Nakurax layers (latent attention and attention beside a recurrence, in turn) beside Zederax and GPT-2 layers. tativik: Tativik "
-                         "layers (windowed latent attention with a rotated key part and a generalized delta rule, in turn, routed experts) beside Nakurax layers")
+                         "layers (windowed latent attention with a rotated key part and a generalized delta rule, in turn, routed experts) beside Nakurax layers. "
+                         "kegetar: Kegetar layers (windowed attention that keeps the first positions beside gated linear attention, and attention whose "
+                         "keys are its values, in turn; dense and routed feed-forwards in turn) beside Tativik layers")
     ap.add_argument("--sizes", default="1k,2k,4k", help="with --workload zederax / nakurax: which of the sizes 1k, 2k, 4k to run")
     ap.add_argument("--batches", default="1,8,64", help="with --workload zederax: decode batch sizes to time ('' for none)")
     ap.add_argument("--no-prefill", action="store_true", help="with --workload zederax: skip the 2,048-token prompt")
-    ap.add_argument("--arch", default="both", choices=["both", "zederax", "gpt2", "nakurax", "tativik"],
+    ap.add_argument("--arch", default="both", choices=["both", "zederax", "gpt2", "nakurax", "tativik", "kegetar"],
                     help="with --workload zederax / nakurax: one architecture only (for profiling)")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -76,7 +78,7 @@ def main() -> int:
     from levanter_amd.config import InferenceEngineConfig, LmConfig
     from levanter_amd.engine import InferenceEngine, Request
 
-    if args.workload in ("zederax", "nakurax", "tativik"):
+    if args.workload in ("zederax", "nakurax", "tativik", "kegetar"):
         return zederax_workload(args)
     if args.workload != "decode":
         return serving_workload(args)
@@ -362,6 +364,30 @@ def tativik_config(z):
     return {"architecture": "Tativik", "vocab": ZEDERAX_VOCAB, "width": z["width"], "norm": {"eps": 1e-6, "groups": 2}, "residual_mult": 0.7, "layers": layers}
 
 
+def kegetar_config(z):
+    """Layers of a windowed rotary attention (the first 64 positions stay in sight, stretched frequencies, a gate per element) beside a
+    gated linear attention with heads of the size's key and value sizes, and layers of an attention whose keys are its values with a
+    distance term, in turn; the heads, head sizes, window and layer count of the size. The feed-forwards are in turn a dense gated one
+    of two thirds of the size's inner width (three matrices hold what the size's two hold) and 30 experts of a quarter of that width
+    beside 2 router outputs that return their input, in 8 groups of which 4 are kept, 4 a token, and a shared expert of the same width."""
+    import math
+
+    left = {"heads": z["heads"], "kv_heads": z["kv_heads"], "dim": z["dim"], "vdim": z["vdim"], "scale": 1.0 / math.sqrt(z["dim"]),
+            "mask": {"size": z["window"], "keep_first": 64},
+            "rot": {"dims": z["dim"], "base": 1000000.0, "scaling": {"factor": 4.0, "original": 8192, "fast": 32.0, "slow": 1.0}}}
+    right = {"heads": z["heads"], "dim": z["dim"], "vdim": z["vdim"], "tau": 16.0, "decay_rank": 64}
+    attention = {"heads": z["heads"], "kv_heads": z["kv_heads"], "dim": z["dim"], "vdim": z["dim"], "scale": 1.0 / math.sqrt(z["dim"]), "mask": {"size": z["window"]}}
+    dense = {"kind": "dense", "ff": z["ff"] * 2 // 3 // 256 * 256}
+    moe = {"kind": "moe", "expert": {"ff": z["ff"] // 4, "limit": 7.0}, "router": {"experts": 30, "identity": 2, "top": 4, "groups": {"count": 8, "keep": 4}},
+           "shared": {"ff": z["ff"] // 4, "limit": 7.0}}
+    layers = []
+    for i in range(z["layers"]):
+        mixer = {"type": "parallel", "mixer": {"left": left, "right": right}} if i % 4 < 2 else {"type": "attention", "mixer": attention}
+        layers.append(json.loads(json.dumps({**mixer, "mlp": dense if i % 2 == 0 else moe})))
+    return {"architecture": "Kegetar", "vocab": ZEDERAX_VOCAB, "width": z["width"], "norm": {"eps": 1e-6}, "residual_mult": 0.7,
+            "embedding": {"bigram": {"buckets": 65521, "mul_prev": 31, "mul_cur": 7}}, "layers": layers}
+
+
 def zederax_workload(args) -> int:
     """Prefill (one 2,048-token prompt) and decode (batch 1, 8, 64 after 512-token prompts) through the engine, for Zederax
     (or, with --workload nakurax, Nakurax and Zederax) and for GPT-2 at equal sizes. One JSON line."""
@@ -435,14 +461,17 @@ def zederax_workload(args) -> int:
             archs.insert(0, ("nakurax", nakurax_config(z)))
         if args.workload == "tativik":  # beside the closest model: Nakurax's latent attention and recurrence
             archs = [("tativik", tativik_config(z)), ("nakurax", nakurax_config(z))]
+        if args.workload == "kegetar":  # beside the closest model: Tativik's windowed attention, matrix-state recurrence and experts
+            archs = [("kegetar", kegetar_config(z)), ("tativik", tativik_config(z))]
         for arch, raw in archs:
             if args.arch in ("both", arch):
                 print(f"[bench] {arch} at size {name} ...", file=sys.stderr, flush=True)
                 results[name][arch] = measure(raw)
-    print(json.dumps({"metric": (f"prefill and decode tok/s of Tativik layers beside Nakurax layers of equal width, heads and (per token) inner width" if args.workload == "tativik" else
+    print(json.dumps({"metric": ("prefill and decode tok/s of Kegetar layers beside Tativik layers of equal width, heads and head sizes" if args.workload == "kegetar" else
+                                 f"prefill and decode tok/s of Tativik layers beside Nakurax layers of equal width, heads and (per token) inner width" if args.workload == "tativik" else
                                  f"prefill and decode tok/s of {args.workload.capitalize()} layers beside {'Zederax and ' if args.workload == 'nakurax' else ''}GPT-2 layers of equal width, heads and inner width"),
                       "unit": "tok/s", "n_gpus": 1, "steps": steps, "warmup": warmup, "dtype": "bf16" if args.dtype == "bfloat16" else "fp32",
-                      "data": "synthetic (random weights, uniform-random token ids)", "results": results}), flush=True)
+                      "data": "synthetic (random weights, uniform-random token ids)", "results": results}), flush=True)  # noqa: E501
     return 0
 
 

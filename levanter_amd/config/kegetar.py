@@ -5,8 +5,9 @@ contribution), ``embedding.bigram`` (``buckets``, ``mul_prev``, ``mul_cur``: an 
 added to the token's; absent: none) and ``layers``, a list with one entry per layer: ``type`` (the mixer: "parallel" or
 "attention"), ``mixer`` (its sizes and constants), ``mlp`` (``kind`` "dense" with ``ff``; ``kind`` "moe" with ``expert`` (``ff``,
 ``limit``), ``router`` (``experts``, ``top``, optional ``identity`` and ``groups`` with ``count`` and ``keep``) and optional ``shared``
-(``ff``, ``limit``); or null for a layer without a feed-forward) and optionally ``weights_of``: the index of an earlier layer with
-tensors of its own whose weights this layer runs, with a cache and state of its own. Layers may differ in all of it.
+(``ff``, ``limit``); or null for a layer without a feed-forward) and optionally ``weights_of``: the index of an earlier layer whose
+tensors this layer runs (that layer's own, or those it runs itself), with a cache and state of its own; its sizes must fit those
+tensors. Layers may differ in all of it.
 
 * parallel: ``left`` (an attention: ``heads``, ``kv_heads``, ``dim``, ``vdim``, ``scale``, ``rot`` with ``dims``, ``base`` and optional
   ``scaling`` (``factor``, ``original``, ``fast``, ``slow``), ``mask`` with ``size`` and ``keep_first``) and ``right`` (a linear attention:
@@ -158,11 +159,17 @@ class KegetarConfig(LmConfig):
             _check_mlp(f"layer {i}", layer.get("mlp"))
             src = layer.get("weights_of")
             if src is not None:
-                if not (isinstance(src, int) and not isinstance(src, bool) and 0 <= src < i) or self.layers[src].get("weights_of") is not None:
-                    raise ConfigError(f"kegetar: layer {i}: weights_of must name an earlier layer with tensors of its own, got {src!r}")
-                other = self.layers[src]
-                if other.get("type") != layer["type"] or other.get("mixer") != m or other.get("mlp") != layer.get("mlp"):
-                    raise ConfigError(f"kegetar: layer {i} runs the weights of layer {src}, but their descriptions differ")
+                if not (isinstance(src, int) and not isinstance(src, bool) and 0 <= src < i):
+                    raise ConfigError(f"kegetar: layer {i}: weights_of must name an earlier layer, got {src!r}")
+                other = self.layers[self.owner_of(src)]
+                if other.get("type") != layer["type"] or (other.get("mlp") or {}).get("kind") != (layer.get("mlp") or {}).get("kind"):
+                    raise ConfigError(f"kegetar: layer {i} runs the weights of layer {self.owner_of(src)}, which is of another kind")
+
+    def owner_of(self, i: int) -> int:
+        """The layer whose tensors layer ``i`` runs: itself, or what its ``weights_of`` leads to."""
+        while self.layers[i].get("weights_of") is not None:
+            i = self.layers[i]["weights_of"]
+        return i
 
     @property
     def n_layers(self) -> int:

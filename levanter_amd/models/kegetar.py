@@ -117,11 +117,16 @@ def kegetar_model_spec(cfg: KegetarConfig) -> ModelSpec:
                          "shared": None if shared is None else gated(f"{p}.shared", shared["ff"], "quick_gelu", False, float(shared["limit"]), EXPERT_UP_SHIFT)},
                         tensors, family="feed_forward")
 
+    def same(a: dict, b: dict) -> bool:
+        return all(a.get(key) == b.get(key) for key in ("type", "mixer", "mlp"))
+
     layers, plan, layer_of = [], [], {}
     for i, layer in enumerate(cfg.layers):
-        src = layer.get("weights_of")
-        if src is None:
-            p, m = f"l{i}", layer["mixer"]
+        owner = cfg.owner_of(i)
+        if owner != i and same(layer, cfg.layers[owner]):  # the earlier layer's built parts, a cache unit of its own
+            layer_of[i] = layer_of[owner]
+        else:  # tensors of its own, or the owner's tensors under constants of its own (another window, say): parts of its own
+            p, m = f"l{owner}", layer["mixer"]
             mixer = parallel(f"{p}.mix", m) if layer["type"] == "parallel" else keys_as_values_attention(f"{p}.mix", m)
             parts = {"mixer": mixer, "connect1": connection(f"{p}.norm1")}
             mlp = layer.get("mlp")
@@ -130,8 +135,6 @@ def kegetar_model_spec(cfg: KegetarConfig) -> ModelSpec:
                 parts["connect2"] = connection(f"{p}.norm2")
             layer_of[i] = len(layers)
             layers.append(LayerSpec("post_norm", parts))
-        else:  # the earlier layer's tensors, a cache unit of its own
-            layer_of[i] = layer_of[src]
         plan.append(PlanEntry(layer=layer_of[i], cache=i, writes_cache=True))
 
     emb_tensors = {"table": TensorSpec("embed", (cfg.vocab, d), std=1.0)}

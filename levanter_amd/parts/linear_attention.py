@@ -64,16 +64,16 @@ class GatedLinearAttention(Mixer):
                 raise ValueError(f"gated_linear_attention: {name} must be {list(shape)}, got {list(t.shape)}")
             return t
 
-        # one product for everything that reads h and needs nothing in between: [q | k | v | gate], each part starting at a multiple
-        # of 8 columns; the decay's low-rank map is two small products of its own
+        # one product for everything that reads h: [q | k | v | gate | the decay's inner sums], each part starting at a multiple of 8
+        # columns; the decay's second product (from its inner sums to a 32-bit sum per key channel) is a small product of its own
         self.qk_part, self.vg_part = _pad8(self.qk_cols), _pad8(self.vg_cols)
         rows = []
         for name, n, padded in (("q", self.qk_cols, self.qk_part), ("k", self.qk_cols, self.qk_part), ("v", self.vg_cols, self.vg_part),
                                 ("gate", self.vg_cols, self.vg_part)):
             rows += [f32(f"{name}.weight", (n, D)), torch.zeros(padded - n, D)]
+        rp = self.rank_padded = _pad8(self.rank)
+        rows += [f32("decay_down.weight", (self.rank, D)), torch.zeros(rp - self.rank, D)]
         self.proj = Linear(torch.cat(rows, 0), None, "out_in", env)
-        rp = _pad8(self.rank)
-        self.decay_down = Linear(torch.cat([f32("decay_down.weight", (self.rank, D)), torch.zeros(rp - self.rank, D)], 0), None, "out_in", env)
         self.decay_up = Linear(torch.cat([f32("decay_up.weight", (self.qk_cols, self.rank)), torch.zeros(self.qk_cols, rp - self.rank)], 1),
                                f32("decay_up.bias", (self.qk_cols,)), "out_in", env)
         nw = tensors["norm.weight"].to(torch.float32).cpu().reshape(-1)
@@ -98,17 +98,14 @@ class GatedLinearAttention(Mixer):
         self.out(a, ctx, out=y, may_leave=True)
 
     def attend(self, p: torch.Tensor, ctx: StepContext, unit: CacheUnitView, writes_cache: bool, a: torch.Tensor, h: torch.Tensor = None) -> None:
-        """Everything between the two products: ``p`` ``[T, q | k | v | gate (| columns of others)]`` is what ``proj`` gives, ``h`` the
-        mixer's input (for the decay's own products), ``a`` ``[T, H*dv]`` takes what ``out`` reads. The request's state is read and
-        advanced."""
+        """Everything between the two products: ``p`` ``[T, q | k | v | gate | decay's inner sums (| columns of others)]`` is what ``proj``
+        gives, ``a`` ``[T, H*dv]`` takes what ``out`` reads. The request's state is read and advanced."""
         if not writes_cache:
             raise ValueError("gated_linear_attention: a recurrence cannot read another entry's state without advancing it")
-        if h is None:
-            raise ValueError("gated_linear_attention: the decay's products need the mixer's input")
-        o1, o2, o3 = self.qk_part, 2 * self.qk_part, 2 * self.qk_part + self.vg_part
+        o1, o2, o3, o4 = self.qk_part, 2 * self.qk_part, 2 * self.qk_part + self.vg_part, 2 * self.qk_part + 2 * self.vg_part
         q, k = p[:, :self.qk_cols], p[:, o1:o1 + self.qk_cols]
         v, g = p[:, o2:o2 + self.vg_cols], p[:, o3:o3 + self.vg_cols]
-        z = self.decay_up(self.decay_down(h, ctx), ctx, out_dtype=torch.float32)
+        z = self.decay_up(p[:, o4:o4 + self.rank_padded], ctx, out_dtype=torch.float32)
         # a step with prompt portions has fewer runs than tokens (at most one per request of the step): the path for prompts
         max_runs = int(ctx.seq_slots.numel()) if ctx.attention.n_prefill_tiles else None
         ctx.kernels.gated_linear_attention(q, k, v, g, z, self.norm_weight, unit.state, ctx.token_slots, a, self.n_heads, self.key_dim, self.value_dim,

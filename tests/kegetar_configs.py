@@ -33,4 +33,17 @@ KEG = {
                          right=P.right_sizes(heads=2, dim=16, vdim=32, tau=16.0, decay_rank=8),
                          mlp=P.experts_mlp(ff=8, experts=2, top=3, identity=1, groups=None, shared=None)),
     ]), 13),
+    # a width that is no multiple of 8, a vocabulary smaller than the width's square root would suggest, a layer that runs the weights of a
+    # layer that runs another's
+    "D": (P.make_config(vocab=50, width=36, bigram=(13, 2, 9), layers=[
+        P.parallel_layer(left=P.left_sizes(heads=2, kv_heads=1, dim=16, vdim=8, window=12, keep_first=2, rot_dims=4),
+                         right=P.right_sizes(heads=1, dim=8, vdim=8, tau=5.0, decay_rank=2), mlp=P.experts_mlp(ff=10, experts=3, top=2, identity=1, groups=(2, 2), shared=6)),
+        P.attention_layer(heads=2, kv_heads=1, dim=8, window=6, mlp=P.dense_mlp(ff=14)),
+        P.parallel_layer(left=P.left_sizes(heads=2, kv_heads=1, dim=16, vdim=8, window=12, keep_first=2, rot_dims=4),
+                         right=P.right_sizes(heads=1, dim=8, vdim=8, tau=5.0, decay_rank=2), mlp=P.experts_mlp(ff=10, experts=3, top=2, identity=1, groups=(2, 2), shared=6),
+                         weights_of=0),
+        P.parallel_layer(left=P.left_sizes(heads=2, kv_heads=1, dim=16, vdim=8, window=12, keep_first=2, rot_dims=4),
+                         right=P.right_sizes(heads=1, dim=8, vdim=8, tau=5.0, decay_rank=2), mlp=P.experts_mlp(ff=10, experts=3, top=2, identity=1, groups=(2, 2), shared=6),
+                         weights_of=2),
+    ]), 14),
 }

@@ -255,8 +255,10 @@ def forward(tokens: List[int], weights: Dict[str, torch.Tensor], cfg: dict) -> T
     streams = []
     margin = torch.full((len(tokens),), math.inf, dtype=F64)
     for i, layer in enumerate(cfg["layers"]):
-        src = layer.get("weights_of")
-        p = f"l{i if src is None else src}"
+        owner = i
+        while cfg["layers"][owner].get("weights_of") is not None:  # whose tensors the layer runs
+            owner = cfg["layers"][owner]["weights_of"]
+        p = f"l{owner}"
         m = layer["mixer"]
         if layer["type"] == "parallel":
             y = parallel_mixer(x, weights, f"{p}.mix", m, eps)

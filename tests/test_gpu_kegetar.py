@@ -450,7 +450,7 @@ def row_error(got, want):
     return (d.pow(2).mean(-1).sqrt() / want.std(-1)).max().item()
 
 
-LENGTHS = {"A": [70, 45, 100, 37, 64, 33], "B": [90, 130, 41, 200, 64, 17], "C": [40, 12, 150, 3]}
+LENGTHS = {"A": [70, 45, 100, 37, 64, 33], "B": [90, 130, 41, 200, 64, 17], "C": [40, 12, 150, 3], "D": [33, 50, 21, 64, 80]}
 
 
 @pytest.mark.parametrize("name", list(KEG))

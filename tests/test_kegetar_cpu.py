@@ -40,7 +40,7 @@ def close(got: torch.Tensor, want: torch.Tensor) -> None:
     assert float(bad) <= 0.01, f"{float(bad):.3%} of the elements differ by more than 2e-4"
 
 
-LENGTHS = {"A": [70, 45, 100, 37, 64, 33], "B": [90, 130, 41, 17, 64], "C": [40, 12, 90]}
+LENGTHS = {"A": [70, 45, 100, 37, 64, 33], "B": [90, 130, 41, 17, 64], "C": [40, 12, 90], "D": [33, 50, 21, 64]}
 
 
 @pytest.fixture(scope="module", params=list(KEG))
@@ -103,6 +103,15 @@ def test_the_registry_finds_the_architecture_and_a_layer_may_run_anothers_weight
     assert reqs[-1] == SlotState((1,), "int32")  # the token before a step's first, kept by the embedding
     # the inner size of the decay's map is what the tensors say: the written configuration does not name it
     assert "decay_rank" not in config.layers[0]["mixer"]["right"] and model.blocks[0].mixer.branches[1].rank == 4
+    # a layer may run a layer that runs another's, and under constants of its own (another window) it gets parts of its own on the same tensors
+    chain = copy.deepcopy(raw)
+    chain["layers"].append(copy.deepcopy(chain["layers"][4]))
+    chain["layers"][6]["weights_of"] = 4
+    chain["layers"][6]["mixer"]["left"]["mask"] = {"size": 11, "keep_first": 2}
+    spec = LmConfig.from_dict(chain).model_spec()
+    assert [e.layer for e in spec.plan] == [0, 1, 2, 3, 0, 3, 4] and len(spec.layers) == 5
+    assert spec.layers[4].mixer.params["left"].params["window"] == 11 and spec.layers[4].mixer.params["left"].tensors["q.weight"].name == "l0.mix.left.q"
+    assert set(spec.all_tensors()) == set(W)
     # a window that is absent keeps everything, and then there are no first positions to keep
     _, _, model_b, _, _ = build("B", tmp_path)
     assert dict(model_b.cache_requirements())[2].paged() == PagedKv(3, 8, None)
@@ -204,8 +213,8 @@ def test_bad_configurations_and_checkpoints_are_refused(tmp_path):
         lambda c: c["layers"][1]["mlp"]["router"]["groups"].update(count=3),  # 8 router outputs do not split into 3
         lambda c: c["layers"][4].update(weights_of=4),  # itself
         lambda c: c["layers"][4].update(weights_of=5),  # a later layer
-        lambda c: c["layers"][5].update(weights_of=4),  # a layer without tensors of its own
-        lambda c: c["layers"][4].update(weights_of=1),  # another description
+        lambda c: c["layers"][5].update(weights_of=4),  # a layer of the other kind (through the layer it runs itself)
+        lambda c: c["layers"][4].update(weights_of=1),  # another kind of feed-forward
         lambda c: c["embedding"]["bigram"].update(buckets=0),
         lambda c: c.pop("norm"),
         lambda c: c.pop("width"),

@@ -599,15 +599,25 @@ extern "C" int lev_norm_average(float* streams, float* x, const float* w, int n,
 // ------------------------------------------------------------------------------------------
 // The activation of a gated feed-forward between its two products: a row of z holds F gate sums and then F up sums,
 //     out[f] = act(g) * (u + up_shift),   g = z[f], u = z[F + f];   with limit > 0: g = min(g, limit), u = clamp(u, -limit, limit).
-// 32-bit arithmetic; `out` may be the first F columns of `z` (a thread reads both of its inputs before it writes).
+// 32-bit arithmetic; `out` may be the first F columns of `z` (a thread reads both of its inputs before it writes). A workgroup
+// takes 1,024 outputs of a row, four a thread, all eight loads in flight at once (a few rows alone would leave the chip empty).
+#define GLU_PER 4
 template <typename T>
 __global__ void __launch_bounds__(256)
 glu_activate_kernel(const T* __restrict__ z, long z_stride, T* __restrict__ out, long o_stride, int F, int act, float limit, float up_shift) {
-  const int t = blockIdx.x;
-  for (int f = threadIdx.x; f < F; f += 256) {
-    float g = to_float<T>(z[(size_t)t * z_stride + f]), u = to_float<T>(z[(size_t)t * z_stride + F + f]);
-    if (limit > 0.f) g = fminf(g, limit), u = fminf(fmaxf(u, -limit), limit);
-    out[(size_t)t * o_stride + f] = from_float<T>(lev_activate(g, act) * (u + up_shift));
+  const int t = blockIdx.x, f0 = blockIdx.y * (256 * GLU_PER) + threadIdx.x;
+  float g[GLU_PER], u[GLU_PER];
+#pragma unroll
+  for (int i = 0; i < GLU_PER; ++i) {
+    const int f = min(f0 + 256 * i, F - 1);  // loads stand under no condition
+    g[i] = to_float<T>(z[(size_t)t * z_stride + f]);
+    u[i] = to_float<T>(z[(size_t)t * z_stride + F + f]);
+  }
+#pragma unroll
+  for (int i = 0; i < GLU_PER; ++i) {
+    const int f = f0 + 256 * i;
+    if (limit > 0.f) g[i] = fminf(g[i], limit), u[i] = fminf(fmaxf(u[i], -limit), limit);
+    if (f < F) out[(size_t)t * o_stride + f] = from_float<T>(lev_activate(g[i], act) * (u[i] + up_shift));
   }
 }
 
@@ -617,8 +627,10 @@ extern "C" int lev_glu_activate(const void* z, long z_stride, void* out, long o_
   LEV_REQUIRE(act >= 0 && act <= LEV_ACT_LAST && limit >= 0.f, "glu_activate: unknown activation %d or a negative limit", act);
   LEV_REQUIRE(dtype == LEV_F32 || dtype == LEV_BF16, "glu_activate: unknown dtype %d", dtype);
   if (T == 0) return 0;
-  if (dtype == LEV_F32) glu_activate_kernel<float><<<T, 256, 0, stream>>>((const float*)z, z_stride, (float*)out, o_stride, F, act, limit, up_shift);
-  else glu_activate_kernel<bf16_t><<<T, 256, 0, stream>>>((const bf16_t*)z, z_stride, (bf16_t*)out, o_stride, F, act, limit, up_shift);
+  const dim3 grid(T, (F + 256 * GLU_PER - 1) / (256 * GLU_PER));
+  LEV_REQUIRE(grid.y <= 65535, "glu_activate: a row of %d outputs is too wide", F);
+  if (dtype == LEV_F32) glu_activate_kernel<float><<<grid, 256, 0, stream>>>((const float*)z, z_stride, (float*)out, o_stride, F, act, limit, up_shift);
+  else glu_activate_kernel<bf16_t><<<grid, 256, 0, stream>>>((const bf16_t*)z, z_stride, (bf16_t*)out, o_stride, F, act, limit, up_shift);
   return lev_check_launch("glu_activate");
 }
 

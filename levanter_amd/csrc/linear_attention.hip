@@ -96,8 +96,8 @@ gla_tokens_kernel(const T* __restrict__ q, const T* __restrict__ k, long qk_stri
 
 // ---- runs of many tokens (prompt portions) --------------------------------------------------------------------------------
 // (1) per token and head, in parallel over the step: the decay a, k and the scaled q as float32 vectors; (2) the walk, one
-// workgroup per (run, head, GLA_CB state columns) of GLA_CB columns x P parts: thread (part, j) keeps the key channels of its part
-// of column j in registers, the vectors of TB tokens at a time are staged through LDS a block ahead, nothing is summed across
+// workgroup per (run, head, GLA_CB state columns) of GLA_CB columns x P = 16 parts: thread (part, j) keeps the key channels of its part
+// of column j in registers, the vectors of TB tokens at a time (8 to 32) are staged through LDS a block ahead, nothing is summed across
 // threads inside the loop (one barrier a block of tokens), and the parts' sums of o = S^T q go to scratch memory; (3) per token
 // and head, in parallel: o from its parts, the head's norm, the weight and the gate.
 template <typename T>
@@ -115,13 +115,15 @@ gla_prepare_kernel(const T* __restrict__ q, const T* __restrict__ k, long qk_str
 }
 
 #define GLA_CB 32  // state columns of a workgroup of the walk: columns never meet, so a head's columns are split over workgroups
-#define GLA_P 8
+#define GLA_P 16  // parts of a column: a thread's share of a token is a chain of dk / 16 dependent steps, and that chain is the walk's time
 template <typename T, int DKM>
 __global__ void __launch_bounds__(GLA_CB * GLA_P)
 gla_scan_kernel(const float* __restrict__ vec, const T* __restrict__ v, long vg_stride, float* __restrict__ state, const int* __restrict__ token_slots,
                 float* __restrict__ part_o /*[Tn][H][P][dv]*/, int Tn, int H, int dk, int dv) {
-  constexpr int P = GLA_P, NT = GLA_CB * P, IP = DKM / P, TB = 1024 / DKM;  // TB tokens' vectors are staged together
-  __shared__ float s_vec[2][TB][3][DKM];
+  // TB tokens' vectors are staged together (48 KB of LDS in two buffers): a block's loads are asked for when the block before it
+  // starts, and what a block costs is the longer of its arithmetic and that latency, so the blocks are as long as the LDS allows
+  constexpr int P = GLA_P, NT = GLA_CB * P, IP = DKM / P, TB = 2048 / DKM;
+  __shared__ __attribute__((aligned(16))) float s_vec[2][TB][3][DKM];
   __shared__ int s_count[NT];
   __shared__ int s_start;
   const int run = blockIdx.x, h = blockIdx.y, tid = threadIdx.x;
@@ -193,17 +195,26 @@ gla_scan_kernel(const float* __restrict__ vec, const T* __restrict__ v, long vg_
 #pragma unroll
     for (int tt = 0; tt < TB; ++tt) {
       const int t = tb + tt;
-      if (t >= t_end) break;  // the whole workgroup
-      const float* a_s = s_vec[buf][tt][0] + part * IP;
-      const float* k_s = s_vec[buf][tt][1] + part * IP;
-      const float* q_s = s_vec[buf][tt][2] + part * IP;
+      if (t >= t_end) continue;  // the whole workgroup; no early exit, so that the loop unrolls and its arrays stay in registers
+      // a part's share of the three vectors in 16-byte reads (IP is a multiple of 4): the walk's time is its LDS reads
+      const float4* a_s = reinterpret_cast<const float4*>(s_vec[buf][tt][0] + part * IP);
+      const float4* k_s = reinterpret_cast<const float4*>(s_vec[buf][tt][1] + part * IP);
+      const float4* q_s = reinterpret_cast<const float4*>(s_vec[buf][tt][2] + part * IP);
       const float vf = vcur[tt];
-      float o = 0.f;
+      float o0 = 0.f, o1 = 0.f, o2 = 0.f, o3 = 0.f;  // four sums side by side: one chain of IP dependent additions would set the pace
 #pragma unroll
-      for (int ii = 0; ii < IP; ++ii) {
-        S[ii] = fmaf(k_s[ii], vf, a_s[ii] * S[ii]);
-        o = fmaf(S[ii], q_s[ii], o);
+      for (int i4 = 0; i4 < IP / 4; ++i4) {
+        const float4 av = a_s[i4], kv = k_s[i4], qv = q_s[i4];
+        S[4 * i4] = fmaf(kv.x, vf, av.x * S[4 * i4]);
+        S[4 * i4 + 1] = fmaf(kv.y, vf, av.y * S[4 * i4 + 1]);
+        S[4 * i4 + 2] = fmaf(kv.z, vf, av.z * S[4 * i4 + 2]);
+        S[4 * i4 + 3] = fmaf(kv.w, vf, av.w * S[4 * i4 + 3]);
+        o0 = fmaf(S[4 * i4], qv.x, o0);
+        o1 = fmaf(S[4 * i4 + 1], qv.y, o1);
+        o2 = fmaf(S[4 * i4 + 2], qv.z, o2);
+        o3 = fmaf(S[4 * i4 + 3], qv.w, o3);
       }
+      const float o = (o0 + o1) + (o2 + o3);
       if (live) part_o[(((size_t)t * H + h) * P + part) * dv + j] = o;
     }
     if (nb >= t_end) break;

@@ -374,8 +374,8 @@ def kegetar_config(z):
 
     left = {"heads": z["heads"], "kv_heads": z["kv_heads"], "dim": z["dim"], "vdim": z["vdim"], "scale": 1.0 / math.sqrt(z["dim"]),
             "mask": {"size": z["window"], "keep_first": 64},
-            "rot": {"dims": z["dim"], "base": 1000000.0, "scaling": {"factor": 4.0, "original": 8192, "fast": 32.0, "slow": 1.0}}}
-    right = {"heads": z["heads"], "dim": z["dim"], "vdim": z["vdim"], "tau": 16.0, "decay_rank": 64}
+            "rot": {"dims": z["dim"], "base": 500000.0, "scaling": {"factor": 8.0, "original": 4096, "fast": 16.0, "slow": 2.0}}}
+    right = {"heads": z["heads"], "dim": z["dim"], "vdim": z["vdim"], "tau": 8.0, "decay_rank": 64}
     attention = {"heads": z["heads"], "kv_heads": z["kv_heads"], "dim": z["dim"], "vdim": z["dim"], "scale": 1.0 / math.sqrt(z["dim"]), "mask": {"size": z["window"]}}
     dense = {"kind": "dense", "ff": z["ff"] * 2 // 3 // 256 * 256}
     moe = {"kind": "moe", "expert": {"ff": z["ff"] // 4, "limit": 7.0}, "router": {"experts": 30, "identity": 2, "top": 4, "groups": {"count": 8, "keep": 4}},
@@ -384,8 +384,8 @@ def kegetar_config(z):
     for i in range(z["layers"]):
         mixer = {"type": "parallel", "mixer": {"left": left, "right": right}} if i % 4 < 2 else {"type": "attention", "mixer": attention}
         layers.append(json.loads(json.dumps({**mixer, "mlp": dense if i % 2 == 0 else moe})))
-    return {"architecture": "Kegetar", "vocab": ZEDERAX_VOCAB, "width": z["width"], "norm": {"eps": 1e-6}, "residual_mult": 0.7,
-            "embedding": {"bigram": {"buckets": 65521, "mul_prev": 31, "mul_cur": 7}}, "layers": layers}
+    return {"architecture": "Kegetar", "vocab": ZEDERAX_VOCAB, "width": z["width"], "norm": {"eps": 1e-6}, "residual_mult": 0.5,
+            "embedding": {"bigram": {"buckets": 65521, "mul_prev": 1009, "mul_cur": 13}}, "layers": layers}
 
 
 def zederax_workload(args) -> int:

@@ -192,11 +192,9 @@ gla_scan_kernel(const float* __restrict__ vec, const T* __restrict__ v, long vg_
 #pragma unroll
     for (int tt = 0; tt < TB; ++tt) vnext[tt] = to_float<T>(v[(size_t)min(nb + tt, Tn - 1) * vg_stride + vcol]);
     lds_barrier();  // the block's vectors are in s_vec[buf]; the loads in flight are the thread's own and are not waited for
-#pragma unroll
-    for (int tt = 0; tt < TB; ++tt) {
-      const int t = tb + tt;
-      if (t >= t_end) continue;  // the whole workgroup; no early exit, so that the loop unrolls and its arrays stay in registers
-      // a part's share of the three vectors in 16-byte reads (IP is a multiple of 4): the walk's time is its LDS reads
+    // one token of the walk; `tt` is a constant wherever this is called, so the arrays stay in registers
+    auto token = [&](const int tt, const int t) {
+      // a part's share of the three vectors in 16-byte reads (IP is a multiple of 4)
       const float4* a_s = reinterpret_cast<const float4*>(s_vec[buf][tt][0] + part * IP);
       const float4* k_s = reinterpret_cast<const float4*>(s_vec[buf][tt][1] + part * IP);
       const float4* q_s = reinterpret_cast<const float4*>(s_vec[buf][tt][2] + part * IP);
@@ -216,6 +214,14 @@ gla_scan_kernel(const float* __restrict__ vec, const T* __restrict__ v, long vg_
       }
       const float o = (o0 + o1) + (o2 + o3);
       if (live) part_o[(((size_t)t * H + h) * P + part) * dv + j] = o;
+    };
+    if (nb <= t_end) {  // a whole block: no condition between its tokens, so the next token's LDS reads can start under this one's arithmetic
+#pragma unroll
+      for (int tt = 0; tt < TB; ++tt) token(tt, tb + tt);
+    } else {
+#pragma unroll
+      for (int tt = 0; tt < TB; ++tt)
+        if (tb + tt < t_end) token(tt, tb + tt);  // the whole workgroup
     }
     if (nb >= t_end) break;
     // the other buffer was last read in the block before this one, which every thread has left (the barrier above)

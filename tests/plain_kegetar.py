@@ -337,7 +337,7 @@ def experts_mlp(ff=24, experts=6, top=2, identity=2, groups=(2, 1), limit=2.0, s
     return mlp
 
 
-def make_config(vocab=97, width=64, layers=None, eps=1e-5, mult=0.7, bigram=(31, 5, 3)) -> dict:
+def make_config(vocab=97, width=64, layers=None, eps=1e-5, mult=0.6, bigram=(31, 5, 3)) -> dict:
     cfg = {"architecture": "Kegetar", "vocab": vocab, "width": width, "norm": {"eps": eps}, "residual_mult": mult,
            "layers": layers if layers is not None else [parallel_layer(), attention_layer()]}
     if bigram:

@@ -89,15 +89,15 @@ class GatedLinearAttention(Mixer):
 
     def forward(self, h: torch.Tensor, x: torch.Tensor, ctx: StepContext, unit: CacheUnitView, writes_cache: bool) -> None:
         a = ctx.empty(h.shape[0], self.vg_cols)
-        self.attend(self.proj(h, ctx), ctx, unit, writes_cache, a, h)
+        self.attend(self.proj(h, ctx), ctx, unit, writes_cache, a)
         self.out(a, ctx, residual=x, final=True)
 
     def compute(self, h: torch.Tensor, y: torch.Tensor, ctx: StepContext, unit: CacheUnitView, writes_cache: bool) -> None:
         a = ctx.empty(h.shape[0], self.vg_cols)
-        self.attend(self.proj(h, ctx), ctx, unit, writes_cache, a, h)
+        self.attend(self.proj(h, ctx), ctx, unit, writes_cache, a)
         self.out(a, ctx, out=y, may_leave=True)
 
-    def attend(self, p: torch.Tensor, ctx: StepContext, unit: CacheUnitView, writes_cache: bool, a: torch.Tensor, h: torch.Tensor = None) -> None:
+    def attend(self, p: torch.Tensor, ctx: StepContext, unit: CacheUnitView, writes_cache: bool, a: torch.Tensor) -> None:
         """Everything between the two products: ``p`` ``[T, q | k | v | gate | decay's inner sums (| columns of others)]`` is what ``proj``
         gives, ``a`` ``[T, H*dv]`` takes what ``out`` reads. The request's state is read and advanced."""
         if not writes_cache:

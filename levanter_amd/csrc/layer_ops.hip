@@ -193,6 +193,66 @@ extern "C" int lev_head_prepare_write(void* q, long q_stride, int H, const void*
 }
 
 // ------------------------------------------------------------------------------------------
+// The norm with a weight and the rotation of head_prepare_write without the write, in place, for runs of several tokens (the
+// pages are written by kv_write afterwards): one wave per (token, item), items are the H query heads and then the G key heads.
+// The arithmetic is head_prepare_write's, operation for operation, so a key is the same bits whichever of the two kernels made it.
+template <typename T>
+__global__ void __launch_bounds__(64)
+head_norm_rotate_kernel(T* __restrict__ q, long q_stride, int H, T* __restrict__ k, long k_stride, int hd, float eps, int norm_dim,
+                        const float* __restrict__ q_norm_w, const float* __restrict__ k_norm_w, const float* __restrict__ freqs, int n_pairs,
+                        const int* __restrict__ positions, float magnitude) {
+  const int t = blockIdx.x, item = blockIdx.y, lane = threadIdx.x;
+  const bool is_q = item < H;
+  T* row = is_q ? q + (size_t)t * q_stride + (size_t)item * hd : k + (size_t)t * k_stride + (size_t)(item - H) * hd;
+  const bool normalise = norm_dim > 0;
+  float r = 1.0f;
+  if (normalise) {
+    float ss = 0.f;
+    for (int d = lane; d < hd; d += 64) {
+      const float x = to_float<T>(row[d]);
+      ss = fmaf(x, x, ss);
+    }
+    ss = wave_sum(ss);
+    r = 1.0f / sqrtf(ss / (float)norm_dim + eps);
+  }
+  const float pos = freqs ? (float)positions[t] : 0.f;
+  const float* norm_w = is_q ? q_norm_w : k_norm_w;
+  for (int i = lane; i < hd / 2; i += 64) {
+    if (!(normalise || i < n_pairs)) continue;
+    float a = to_float<T>(row[2 * i]), b = to_float<T>(row[2 * i + 1]);
+    if (normalise) a *= r, b *= r;
+    if (normalise && norm_w) a *= norm_w[2 * i], b *= norm_w[2 * i + 1];
+    if (i < n_pairs) {
+      float sn, cs;
+      sincosf(pos * freqs[i], &sn, &cs);
+      sn *= magnitude, cs *= magnitude;
+      const float ra = a * cs - b * sn, rb = b * cs + a * sn;
+      a = ra, b = rb;
+    }
+    row[2 * i] = from_float<T>(a), row[2 * i + 1] = from_float<T>(b);
+  }
+}
+
+extern "C" int lev_head_norm_rotate(void* q, long q_stride, int H, void* k, long k_stride, int G, int hd, float eps, int norm_dim,
+                                    const float* q_norm_w, const float* k_norm_w, const float* freqs, int n_pairs, const int* positions,
+                                    float magnitude, int T, int dtype, hipStream_t stream) {
+  LEV_REQUIRE(T >= 0 && H >= 0 && G >= 0 && hd > 0 && hd % 2 == 0, "head_norm_rotate: bad sizes T=%d heads=%d/%d size=%d", T, H, G, hd);
+  LEV_REQUIRE((H == 0 || q) && (G == 0 || k), "head_norm_rotate: a tensor is missing");
+  LEV_REQUIRE(n_pairs >= 0 && 2 * n_pairs <= hd && (n_pairs == 0 || (freqs && positions)), "head_norm_rotate: %d rotated pairs need frequencies, positions and a head of at least twice their number", n_pairs);
+  LEV_REQUIRE(norm_dim >= 0 && norm_dim <= hd && H + G <= 65535, "head_norm_rotate: the norm's divisor %d must lie in 0 .. %d", norm_dim, hd);
+  LEV_REQUIRE(dtype == LEV_F32 || dtype == LEV_BF16, "head_norm_rotate: unknown dtype %d", dtype);
+  if (T == 0 || H + G == 0) return 0;
+  dim3 grid(T, H + G);
+  if (dtype == LEV_F32)
+    head_norm_rotate_kernel<float><<<grid, 64, 0, stream>>>((float*)q, q_stride, H, (float*)k, k_stride, hd, eps, norm_dim, q_norm_w, k_norm_w, freqs, n_pairs,
+                                                           positions, magnitude);
+  else
+    head_norm_rotate_kernel<bf16_t><<<grid, 64, 0, stream>>>((bf16_t*)q, q_stride, H, (bf16_t*)k, k_stride, hd, eps, norm_dim, q_norm_w, k_norm_w, freqs,
+                                                            n_pairs, positions, magnitude);
+  return lev_check_launch("head_norm_rotate");
+}
+
+// ------------------------------------------------------------------------------------------
 // A row of R values per token that is one key/value head for all query heads (a latent that keys and values are both made
 // from): its RMS norm with a weight, x / sqrt(sum(x^2) / norm_dim + eps) * w, in place, and the result written into the key
 // pages [page][1][R/8][PS][8] and the value pages [page][1][R][PS] at dest[t] = page * PS + offset (negative: nowhere). One

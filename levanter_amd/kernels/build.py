@@ -299,6 +299,7 @@ register_unit("core", ["errors.hip", "elementwise.hip", "layer_ops.hip", "gemm_s
     "lev_kv_write": [_P, _P, _L, _L, _P, _P, _P] + [_I] * 6 + [_P],
     "lev_head_prepare": [_P, _L, _I, _I, _I, _F, _P, _L, _P, _L, _I, _I, _P, _P, _I, _I, _P],
     "lev_head_prepare_write": [_P, _L, _I, _P, _L, _P, _L, _P, _L, _P, _I, _I, _I, _F, _I, _P, _P, _P, _I, _P, _I, _P, _P, _P, _F, _I, _I, _P],
+    "lev_head_norm_rotate": [_P, _L, _I, _P, _L, _I, _I, _F, _I, _P, _P, _P, _I, _P, _F, _I, _I, _P],
     "lev_norm_write_latent": [_P, _L, _I, _I, _F, _P, _P, _P, _P, _I, _I, _I, _P],
     "lev_recurrent_tokens": [_P, _L, _P, _L, _P, _P, _P, _P, _P, _P, _P, _P, _L, _I, _I, _I, _I, _F, _I, _P],
     "lev_poly_norm": [_P, _L, _P, _L, _P, _I, _I, _F, _I, _P],

@@ -513,6 +513,27 @@ class HipKernels:
             _ptr(rotary_freqs) if n_pairs else None, n_pairs, _ptr(positions) if n_pairs else None, _ptr(q_norm_weight), _ptr(k_norm_weight),
             float(rotary_magnitude), T, _DT[dt], self._s()))
 
+    def head_norm_rotate(self, q, k, n_heads: int, n_kv_heads: int, head_dim: int, eps: Optional[float], norm_dim: Optional[int] = None,
+                         q_norm_weight=None, k_norm_weight=None, rotary_freqs=None, positions=None, rotary_magnitude: float = 1.0) -> None:
+        """What ``head_prepare_write`` does to queries and keys, without the write and in place on both: every head divided by its root
+        mean square (``eps`` None: not), times the norm's weight of its kind, then the rotation of ``rotary_pairs``. For runs of
+        several tokens, whose pages ``kv_write`` fills afterwards; the same arithmetic, so a key is the same bits either way."""
+        _dev(q, k, q_norm_weight, k_norm_weight, rotary_freqs, positions)
+        T, dt = q.shape[0], q.dtype
+        _req(dt in _DT and k.dtype == dt and q.shape == (T, n_heads * head_dim) and k.shape == (T, n_kv_heads * head_dim), "head_norm_rotate: q and k must be [T, heads*head_dim] of one compute dtype")
+        for w in (q_norm_weight, k_norm_weight):
+            _req(w is None or (eps is not None and w.dtype == torch.float32 and w.numel() == head_dim and w.is_contiguous()),
+                 "head_norm_rotate: a norm's weight must be float32 [head_dim] and needs the norm")
+        n_pairs = 0
+        if rotary_freqs is not None:
+            _req(rotary_freqs.dtype == torch.float32 and rotary_freqs.is_contiguous() and 2 * rotary_freqs.numel() <= head_dim, "head_norm_rotate: float32 frequencies, at most head_dim / 2")
+            _req(positions is not None and positions.dtype == torch.int32 and positions.numel() == T, "head_norm_rotate: one int32 position per token")
+            n_pairs = rotary_freqs.numel()
+        self._check(self.lib.lev_head_norm_rotate(_ptr(q), _rows(q, "head_norm_rotate: q"), int(n_heads), _ptr(k), _rows(k, "head_norm_rotate: k"), int(n_kv_heads),
+                                                  int(head_dim), float(eps or 0.0), int(norm_dim or head_dim) if eps is not None else 0, _ptr(q_norm_weight),
+                                                  _ptr(k_norm_weight), _ptr(rotary_freqs) if n_pairs else None, n_pairs, _ptr(positions) if n_pairs else None,
+                                                  float(rotary_magnitude), T, _DT[dt], self._s()))
+
     def norm_write_latent(self, c, weight, eps: float, norm_dim: int, k_pages, v_pages, dest, page_size: int) -> None:
         """``c`` ``[T, R]`` (one key/value head that all query heads share) becomes its RMS norm with ``weight`` (float32 ``[R]``;
         the mean of squares is over ``norm_dim``), in place, and goes into the key and the value pages at ``dest``: what

@@ -192,19 +192,21 @@ class TalkingHeadsAttention(Mixer):
             K.head_prepare(q, 1, self.q_cols, self.qk_norm_eps, norm_dim=self.n_heads * self.true_head_dim, norm_weight=self.q_norm_weight)
             K.head_prepare(k, 1, self.k_cols, self.qk_norm_eps, norm_dim=self.n_kv_heads * self.true_head_dim, norm_weight=self.k_norm_weight)
         elif self.qk_norm == "head":
-            if single:  # inside the kernel that writes the pages
-                fused_norm = {"q_norm_weight": self.q_norm_weight, "k_norm_weight": self.k_norm_weight}
-            else:  # a norm with a weight does not commute with the rotation: it comes first
-                K.head_prepare(q, self.n_heads, self.head_dim, self.qk_norm_eps, norm_dim=self.true_head_dim, norm_weight=self.q_norm_weight)
-                K.head_prepare(k, self.n_kv_heads, self.head_dim, self.qk_norm_eps, norm_dim=self.true_head_dim, norm_weight=self.k_norm_weight)
-        if self.rotary is not None:
-            if single and getattr(self.rotary, "freqs", None) is not None and getattr(self.rotary, "head_dim", None) == self.head_dim:
-                # a step of single tokens: the rotation happens inside the kernel that writes the pages
-                fused_rotation = {"rotary_freqs": self.rotary.freqs, "positions": ctx.attention.positions} if self.rotary.freqs.numel() else {}
-                if fused_rotation and getattr(self.rotary, "magnitude", 1.0) != 1.0:
-                    fused_rotation["rotary_magnitude"] = self.rotary.magnitude
-            else:
+            fused_norm = {"q_norm_weight": self.q_norm_weight, "k_norm_weight": self.k_norm_weight}
+        rot_here = self.rotary is not None and getattr(self.rotary, "freqs", None) is not None and getattr(self.rotary, "head_dim", None) == self.head_dim
+        if self.rotary is not None and rot_here and (single or fused_norm):
+            # a step of single tokens: the rotation happens inside the kernel that writes the pages; with a weighted norm ahead of it,
+            # a step with longer runs does both in one kernel of the same arithmetic (a norm with a weight does not commute with the rotation)
+            fused_rotation = {"rotary_freqs": self.rotary.freqs, "positions": ctx.attention.positions} if self.rotary.freqs.numel() else {}
+            if fused_rotation and getattr(self.rotary, "magnitude", 1.0) != 1.0:
+                fused_rotation["rotary_magnitude"] = self.rotary.magnitude
+        if fused_norm and (not single or (self.rotary is not None and not rot_here)):
+            K.head_norm_rotate(q, k, self.n_heads, self.n_kv_heads, self.head_dim, self.qk_norm_eps, norm_dim=self.true_head_dim, **fused_norm, **fused_rotation)
+            if self.rotary is not None and not rot_here:  # a rotation of another kind: behind the norm
                 self.rotary.rotate(q, k, ctx)
+            fused_norm, fused_rotation = {}, {}  # both are done: what writes the pages only writes
+        elif self.rotary is not None and not (single and rot_here):
+            self.rotary.rotate(q, k, ctx)
         v_first = None
         if self.value_mix == "source":
             ctx.shared[self.value_mix_key] = v

@@ -465,6 +465,14 @@ class EmulatedKernels:
             self.head_prepare(None, 0, 0, 0.0, v=v, v_first=v_first, n_blend=n_kv_heads, value_dim=value_dim, blend=blend)
         self.kv_write(k, v, k_pages, v_pages, dest, n_kv_heads, head_dim, page_size, value_dim=value_dim)
 
+    def head_norm_rotate(self, q, k, n_heads, n_kv_heads, head_dim, eps, norm_dim=None, q_norm_weight=None, k_norm_weight=None, rotary_freqs=None,
+                         positions=None, rotary_magnitude=1.0) -> None:
+        if eps is not None:
+            self.head_prepare(q, n_heads, head_dim, eps, norm_dim=norm_dim, norm_weight=q_norm_weight)
+            self.head_prepare(k, n_kv_heads, head_dim, eps, norm_dim=norm_dim, norm_weight=k_norm_weight)
+        if rotary_freqs is not None:
+            self.rotary_pairs(q, k, head_dim, rotary_freqs, positions, rotary_magnitude)
+
     def norm_write_latent(self, c, weight, eps, norm_dim, k_pages, v_pages, dest, page_size) -> None:
         self.head_prepare(c, 1, c.shape[1], eps, norm_dim=norm_dim, norm_weight=weight)
         self.kv_write(c, c, k_pages, v_pages, dest, 1, c.shape[1], page_size)

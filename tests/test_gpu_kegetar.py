@@ -141,6 +141,30 @@ def test_norm_with_weights_rotation_and_write_of_single_tokens_in_one_kernel_is_
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("H,G,hd,vd,n_pairs", [(4, 2, 16, 8, 8), (2, 2, 32, 32, 4), (3, 1, 64, 16, 32), (1, 1, 8, 24, 0), (2, 1, 160, 16, 80)])
+def test_norm_and_rotation_of_a_run_are_those_of_single_tokens_bit_for_bit(dtype, H, G, hd, vd, n_pairs):
+    """A key is the same bits whether its token came in a prompt's portion or alone."""
+    g = torch.Generator().manual_seed(hd + vd)
+    T, ps = 6, 16
+    q, k, v = (torch.randn(T, n, generator=g).to(dtype).to(DEV) for n in (H * hd, G * hd, G * vd))
+    wq, wk = (1.5 + torch.randn(hd, generator=g) * 0.3).to(DEV), (1.5 + torch.randn(hd, generator=g) * 0.3).to(DEV)
+    freqs = torch.rand(n_pairs, generator=g).to(DEV)
+    pos = ints([3, 0, 700, 15, 16, 4000])
+    dest = ints([5, 17, 33, 40, 3 * ps + 15, 0])
+    kp1, vp1 = torch.zeros(4, G * hd * ps, dtype=dtype, device=DEV), torch.zeros(4, G * vd * ps, dtype=dtype, device=DEV)
+    kp2, vp2 = torch.zeros_like(kp1), torch.zeros_like(vp1)
+    rot = {"rotary_freqs": freqs, "positions": pos, "rotary_magnitude": 1.1} if n_pairs else {}
+    q1 = q.clone()
+    K().head_prepare_write(q1, k, v, kp1, vp1, dest, H, G, hd, vd, ps, 1e-5, q_norm_weight=wq, k_norm_weight=wk, **rot)
+    q2, k2 = q.clone(), k.clone()
+    K().head_norm_rotate(q2, k2, H, G, hd, 1e-5, q_norm_weight=wq, k_norm_weight=wk, **rot)
+    K().kv_write(k2, v, kp2, vp2, dest, G, hd, ps, value_dim=vd)
+    assert torch.equal(q1.cpu(), q2.cpu()) and torch.equal(kp1.cpu(), kp2.cpu()) and torch.equal(vp1.cpu(), vp2.cpu())
+    want = P.rotate_pairs(P.rms_norm(k.cpu().double().view(T, G, hd), wk.cpu().double(), 1e-5), pos.cpu(), freqs.cpu().double().tolist(), 1.1 if n_pairs else 1.0)
+    torch.testing.assert_close(k2.cpu().double().view(T, G, hd), want, **(dict(rtol=3e-3, atol=3e-3) if dtype == torch.float32 else dict(rtol=3e-2, atol=3e-2)))
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
 def test_a_gate_per_element_of_the_heads(dtype):
     g = torch.Generator().manual_seed(1)
     T, H, vd = 5, 3, 24
